@@ -204,6 +204,81 @@ def load() -> ctypes.CDLL:
     return lib
 
 
+# ---- libi64hip_dense.so (include/i64h_dense.h) -------------------------------------------------------------------------------------
+DENSE_LIB_PATH = os.path.join(_HERE, "libi64hip_dense.so")
+DENSE_SIGNATURES: Dict[str, str] = {
+    "i64h_linear_run": "pp",
+    "i64h_set_linear_skinny": "i",
+    "i64h_embed_scaled": "ppfplilp",
+    "i64h_gated_postnorm": "pp",
+    "i64h_latent_prep": "pp",
+    "i64h_latent_attn": "pp",
+    "i64h_sample_rows": "pplippppp",
+}
+
+
+class Linear(ctypes.Structure):
+    """Mirror of i64h_linear (include/i64h_dense.h)."""
+    _fields_ = [("A", _P), ("lda", _L), ("a_rows", _P), ("W", _P), ("C", _P), ("ldc", _L), ("M", _L), ("N", _I), ("K", _I), ("batch", _I),
+                ("a_batch", _L), ("w_batch", _L), ("c_batch", _L), ("exact", _I), ("epilogue", _I), ("E", _P), ("lde", _L), ("e_batch", _L),
+                ("softcap", _F)]
+
+
+class PostNorm(ctypes.Structure):
+    """Mirror of i64h_postnorm (include/i64h_dense.h)."""
+    _fields_ = [("x", _P), ("x_rows", _P), ("y", _P), ("ldy", _L), ("gate_pre", _P), ("ldg", _L), ("gate_bias", _P), ("alpha", _F),
+                ("norm_w", _P), ("groups", _I), ("eps", _F), ("out", _P), ("hist", _P), ("hist_index", _I), ("mix_w", _P), ("mix_out", _P),
+                ("n", _L), ("W", _I)]
+
+
+class LatentPrep(ctypes.Structure):
+    """Mirror of i64h_latent_prep_args (include/i64h_dense.h)."""
+    _fields_ = [("P", _P), ("ldp", _L), ("q_off", _I), ("dkv_off", _I), ("heads", _I), ("dim", _I), ("rot_dim", _I), ("kv_rank", _I),
+                ("rot_dims", _I), ("c_norm_w", _P), ("eps", _F), ("inv_freq", _P), ("positions", _P), ("slot_ids", _P), ("block_table", _P),
+                ("max_blocks_per_seq", _I), ("block_size", _I), ("cache", _P), ("cache_dtype", _I), ("Q", _P), ("n", _L)]
+
+
+class LatentAttn(ctypes.Structure):
+    """Mirror of i64h_latent_attn_args (include/i64h_dense.h)."""
+    _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
+                ("slot_ids", _P), ("positions", _P), ("window", _I), ("scale", _F), ("out", _P), ("n", _L), ("heads", _I), ("kv_rank", _I),
+                ("rot_dim", _I), ("mode", _I)]
+
+
+_dense: Optional[ctypes.CDLL] = None
+
+
+def dense_exported_symbols():
+    return ["i64h_last_error", "i64h_version", "i64h_device_check", *DENSE_SIGNATURES.keys()]
+
+
+def load_dense() -> ctypes.CDLL:
+    """Load libi64hip_dense.so once; raises if it has not been built (no CPU fallback exists)."""
+    global _dense
+    if _dense is not None:
+        return _dense
+    import torch  # noqa: F401  (one HIP runtime per process: torch's)
+    if not os.path.exists(DENSE_LIB_PATH):
+        raise I64HError(f"{DENSE_LIB_PATH} not found: build it with `python vllm_i64_amd/build.py --dense-only` (no CPU fallback exists)")
+    lib = ctypes.CDLL(DENSE_LIB_PATH)
+    lib.i64h_last_error.restype = ctypes.c_char_p
+    lib.i64h_last_error.argtypes = []
+    lib.i64h_device_check.restype = _I
+    for name, sig in DENSE_SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = _I
+        fn.argtypes = [_KIND[c] for c in sig]
+    _dense = lib
+    return lib
+
+
+def call_dense(name: str, *args):
+    lib = load_dense()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise I64HError(f"{name} failed ({rc}): {lib.i64h_last_error().decode()}")
+
+
 def ptr(t) -> int:
     """Device (or host) address of a tensor / ctypes buffer; None -> NULL."""
     if t is None:

@@ -1,4 +1,9 @@
-"""Build libi64hip.so (gfx950 code objects + C ABI) in-tree with hipcc.  No GPU needed: hipcc cross-compiles."""
+"""Build the in-tree HIP libraries (gfx950 code objects + C ABI) with hipcc.  No GPU needed: hipcc cross-compiles.
+
+libi64hip.so        the quantized token-routed-MoE forward (include/i64h.h)
+libi64hip_dense.so  models with bf16 weights and a 32-bit residual: Linear, gated post-norm, latent attention, sampling
+                    (include/i64h_dense.h) - a library of its own, so that serving such a model builds nothing else
+"""
 from __future__ import annotations
 
 import os
@@ -9,10 +14,14 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libi64hip.so")
+DENSE_OUT = os.path.join(HERE, "libi64hip_dense.so")
+DENSE_SOURCES = ["i64h_api.hip", "i64h_dense.hip", "i64h_latent.hip"]
 SOURCES = ["i64h_api.hip", "i64h_route.hip", "i64h_quant.hip", "i64h_norm.hip", "i64h_gemm.hip", "i64h_gemm_os.hip", "i64h_attn.hip", "i64h_moe.hip", "i64h_fp8.hip", "i64h_kv.hip", "i64h_decode.hip", "i64h_variants.hip", "i64h_group_f32.hip", "i64h_lmhead.hip"]
 # -ffp-contract=off: a*b+c stays two roundings unless the source says fmaf, so fp32 element-wise math has the
 # same rounding steps as the reference's CPU ops.
+# no packed-fp32 instructions: the compiler forms them from ordinary float code, and some of their forms have been unreliable
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-ffp-contract=off", "-Wall", "-Wno-unused-function",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
          "-I", os.path.join(os.path.dirname(HERE), "include"), "-I", CSRC]
 
 
@@ -31,12 +40,13 @@ def _stale(obj: str, src: str) -> bool:
     return any(os.path.getmtime(d) > t for d in deps)
 
 
-def build(force: bool = False, verbose: bool = True) -> str:
+def build(force: bool = False, verbose: bool = True, sources=None, out: str = OUT) -> str:
+    sources = SOURCES if sources is None else sources
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     jobs = []
-    for s in SOURCES:
+    for s in sources:
         src = os.path.join(CSRC, s)
         obj = os.path.join(objdir, s.replace(".hip", ".o"))
         if force or _stale(obj, src):
@@ -48,19 +58,27 @@ def build(force: bool = False, verbose: bool = True) -> str:
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"hipcc failed: {' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
-        if verbose and r.stderr.strip():
-            print(r.stderr.strip())
+        # (the host pass does not know the device-only feature switch and says so once per function: not worth a line each)
+        noise = [ln for ln in r.stderr.splitlines() if ln.strip() and "is not a recognized feature for this target" not in ln]
+        if verbose and noise:
+            print("\n".join(noise))
 
     with ThreadPoolExecutor(max_workers=min(6, max(1, len(jobs)))) as ex:
         list(ex.map(run, jobs))
-    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in SOURCES]
-    if jobs or not os.path.exists(OUT):
-        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", OUT]
+    objs = [os.path.join(objdir, s.replace(".hip", ".o")) for s in sources]
+    if jobs or not os.path.exists(out):
+        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
-    return OUT
+    return out
+
+
+def build_dense(force: bool = False, verbose: bool = True) -> str:
+    return build(force=force, verbose=verbose, sources=DENSE_SOURCES, out=DENSE_OUT)
 
 
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv))
+    if "--dense-only" not in sys.argv:
+        print(build(force="--force" in sys.argv))
+    print(build_dense(force="--force" in sys.argv))

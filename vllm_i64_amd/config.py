@@ -72,3 +72,115 @@ def trmoe306_synth() -> ModelConfig:
 def dense306_synth() -> ModelConfig:
     return ModelConfig(name="dense306-synth", num_layers=18, intermediate_size=4096, num_experts=1, shared_intermediate_size=0,
                        top_k=1, primary_weight=1.0, table_routing=False)
+
+
+# ---------------------------------------------------------------------------------------------------------------------------
+# Morilorn: post-norm decoder with gated residuals, grouped RMS norm, depth mixing and latent attention.  Every size and every
+# constant comes from the checkpoint's config.json; layers are listed one by one and may differ from each other.
+# ---------------------------------------------------------------------------------------------------------------------------
+@dataclass
+class LatentAttentionConfig:
+    heads: int
+    dim: int                 # unrotated query / key dimensions per head
+    rot_dim: int             # rotated query / key dimensions per head (the key part is shared by all heads)
+    vdim: int                # value dimensions per head
+    kv_rank: int             # width of the cached latent
+    scale: float             # multiplies the scores
+    window: int = 0          # a position sees itself and the window - 1 before it; 0: all earlier positions
+    rot_base: float = 10000.0
+    rot_dims: int = 0        # leading dimensions of the rotated part that are rotated (the rest pass through)
+
+    @property
+    def q_width(self) -> int:
+        return self.heads * (self.dim + self.rot_dim)
+
+    @property
+    def cache_width(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "LatentAttentionConfig":
+        rot = m.get("rot") or {}
+        rot_dim = int(m.get("rot_dim", 0))
+        mask = m.get("mask") or {}
+        c = cls(heads=int(m["heads"]), dim=int(m["dim"]), rot_dim=rot_dim, vdim=int(m["vdim"]), kv_rank=int(m["kv_rank"]),
+                scale=float(m["scale"]), window=int(mask.get("size", 0)), rot_base=float(rot.get("base", 10000.0)),
+                rot_dims=int(rot.get("dims", rot_dim)) if rot_dim else 0)
+        if c.rot_dims > c.rot_dim or c.rot_dims % 2:
+            raise ValueError(f"latent_attention: {c.rot_dims} rotated dimensions do not fit a rotated part of {c.rot_dim}")
+        if min(c.heads, c.dim, c.vdim, c.kv_rank) <= 0 or c.window < 0:
+            raise ValueError(f"latent_attention: bad sizes {m}")
+        return c
+
+
+@dataclass
+class DenseMlpConfig:
+    ff: int
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "DenseMlpConfig":
+        if m.get("kind", "dense") != "dense":
+            raise ValueError(f"feed-forward kind '{m.get('kind')}' is not built")
+        return cls(ff=int(m["ff"]))
+
+
+MIXERS = {"latent_attention": LatentAttentionConfig}
+
+
+@dataclass
+class DecoderLayerConfig:
+    type: str
+    mixer: LatentAttentionConfig
+    mlp: "DenseMlpConfig | None"
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "DecoderLayerConfig":
+        kind = d.get("type")
+        if kind not in MIXERS:
+            raise ValueError(f"layer type '{kind}' is not built (known: {sorted(MIXERS)})")
+        mlp = d.get("mlp")
+        return cls(type=kind, mixer=MIXERS[kind].from_dict(d["mixer"]), mlp=DenseMlpConfig.from_dict(mlp) if mlp else None)
+
+
+@dataclass
+class MorilornConfig:
+    vocab: int
+    width: int
+    layers: list
+    embedding_scale: float = 1.0
+    postln_alpha: float = 1.0
+    norm_eps: float = 1e-6
+    norm_groups: int = 1
+    logit_softcap: float = 0.0     # 0: logits are not capped
+    name: str = "Morilorn"
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "MorilornConfig":
+        norm = d.get("norm") or {}
+        c = cls(vocab=int(d["vocab"]), width=int(d["width"]), layers=[DecoderLayerConfig.from_dict(l) for l in d["layers"]],
+                embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)), postln_alpha=float(d.get("postln_alpha", 1.0)),
+                norm_eps=float(norm.get("eps", 1e-6)), norm_groups=int(norm.get("groups", 1)), logit_softcap=float(d.get("logit_softcap") or 0.0),
+                name=str(d.get("architecture", "Morilorn")))
+        if c.width % c.norm_groups:
+            raise ValueError(f"width {c.width} does not split into {c.norm_groups} norm groups")
+        return c
+
+    def to_dict(self) -> dict:
+        layers = []
+        for l in self.layers:
+            m = l.mixer
+            mixer = {"heads": m.heads, "dim": m.dim, "rot_dim": m.rot_dim, "vdim": m.vdim, "kv_rank": m.kv_rank, "scale": m.scale,
+                     "rot": {"base": m.rot_base, "dims": m.rot_dims}}
+            if m.window:
+                mixer["mask"] = {"size": m.window}
+            layers.append({"type": l.type, "mixer": mixer, "mlp": {"kind": "dense", "ff": l.mlp.ff} if l.mlp else None})
+        return {"architecture": "Morilorn", "vocab": self.vocab, "width": self.width, "layers": layers, "embedding": {"scale": self.embedding_scale},
+                "postln_alpha": self.postln_alpha, "norm": {"eps": self.norm_eps, "groups": self.norm_groups}, "logit_softcap": self.logit_softcap}

@@ -95,41 +95,9 @@ def pack_fp8(w: torch.Tensor, device) -> PackedFp8:
     return PackedFp8(q.view(G, N, K), s.view(G, N))
 
 
-# ---------------------------------------------------------------------------------------------------------
-# paged KV cache: reference layout (num_blocks, 16, kv_heads, head_dim) + int32 block table (core/kv_cache.py:84-107)
-# ---------------------------------------------------------------------------------------------------------
-class PagedKVCache:
-    def __init__(self, cfg: ModelConfig, num_blocks: int, max_seqs: int, device, dtype=torch.float32):
-        self.cfg, self.block, self.device, self.dtype = cfg, cfg.kv_block, device, dtype
-        shape = (num_blocks, cfg.kv_block, cfg.num_kv_heads, cfg.head_dim)
-        self.k = [torch.zeros(shape, dtype=dtype, device=device) for _ in range(cfg.num_layers)]
-        self.v = [torch.zeros(shape, dtype=dtype, device=device) for _ in range(cfg.num_layers)]
-        self.max_blocks_per_seq = (cfg.max_pos + cfg.kv_block - 1) // cfg.kv_block
-        self._bt_host = torch.full((max_seqs, self.max_blocks_per_seq), -1, dtype=torch.int32)
-        self.block_table = self._bt_host.to(device)
-        self._free = list(range(num_blocks - 1, -1, -1))
-        self._owned: Dict[int, int] = {}
-
-    def reserve(self, slot: int, length: int):
-        """Make sure sequence `slot` owns blocks for positions [0, length). Host bookkeeping + one small upload."""
-        need = (length + self.block - 1) // self.block
-        have = self._owned.get(slot, 0)
-        if need <= have:
-            return
-        if need > self.max_blocks_per_seq:
-            raise RuntimeError(f"sequence length {length} exceeds max_pos {self.cfg.max_pos}")
-        if need - have > len(self._free):
-            raise RuntimeError("paged KV cache exhausted")
-        for b in range(have, need):
-            self._bt_host[slot, b] = self._free.pop()
-        self._owned[slot] = need
-        self.block_table[slot].copy_(self._bt_host[slot], non_blocking=True)
-
-    def free(self, slot: int):
-        for b in range(self._owned.pop(slot, 0)):
-            self._free.append(int(self._bt_host[slot, b]))
-            self._bt_host[slot, b] = -1
-        self.block_table[slot].copy_(self._bt_host[slot], non_blocking=True)
+# the paged KV cache (reference layout (num_blocks, 16, kv_heads, head_dim) + int32 block table) lives beside the package's other
+# cache layouts, on the shared page pool
+from .paged_cache import PagedKVCache  # noqa: E402,F401
 
 
 # ---------------------------------------------------------------------------------------------------------
