@@ -60,6 +60,10 @@ def parse():
                          "(e4m3fn weights per output channel, e4m3fn activations per token) on the fp8 matrix cores")
     ap.add_argument("--no-replica-leg", action="store_true",
                     help="N > 1: skip the second, labelled measurement of independent replicas (reported beside the expert-parallel value)")
+    ap.add_argument("--design", default="", choices=["", "morilorn"],
+                    help="instead of the headline workload: prefill / decode throughput of another registered design at real layer sizes beside "
+                         "the closest existing model, and its kernels against their rooflines (vllm_i64_amd/bench_designs.py)")
+    ap.add_argument("--design-sizes", default="", help="--design: sizes to run, with commas between them (default: all)")
     return ap.parse_args()
 
 
@@ -112,6 +116,9 @@ def cpu_baseline(cfg, weights, batch, ctx, steps, mode="int8_torch"):
 
 def main():
     args = parse()
+    if args.design:
+        from vllm_i64_amd import bench_designs
+        raise SystemExit(bench_designs.main(args))
     rank = int(os.environ.get("RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))

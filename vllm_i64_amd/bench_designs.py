@@ -1,0 +1,187 @@
+"""`bench.py --design morilorn`: prefill and decode throughput of the Morilorn design at layer sizes of real models (random weights),
+beside the package's closest existing model (the dense int8 decoder) at equal width, depth, feed-forward size and batch, and the
+design's kernels one by one against their rooflines beside the like kernel of that model.  Prints one JSON line."""
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+HBM_GBS, BF16_TFLOPS, I8_TOPS = 8000.0, 2500.0, 5000.0      # MI355X: HBM3E, dense bf16 and dense int8 matrix-core peaks
+
+SIZES = {
+    "w1024": dict(width=1024, layers=18, heads=16, dim=32, rot_dim=32, vdim=64, kv_rank=256, ff=4096, window=1024, kv_heads=4),
+    "w2048": dict(width=2048, layers=8, heads=32, dim=32, rot_dim=32, vdim=64, kv_rank=512, ff=8192, window=1024, kv_heads=8),
+}
+
+
+def _time(fn, reps: int, warm: int = 3) -> float:
+    """Seconds per call, device time between two events around `reps` back-to-back calls."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps * 1e-3
+
+
+def _steps(model, dec_cls, batch, ctx, prefill_rows, prefill_seq, steps, warmup, fill, vocab, dev):
+    """(prefill tokens/s, decode tokens/s, decode ms/step): one prefill step of prefill_rows rows (sequences of prefill_seq tokens), then a
+    batch of `batch` sequences at context ctx (cache contents synthetic) decoding greedily, the step replayed as a HIP graph."""
+    g = torch.Generator().manual_seed(3)
+    nseq = prefill_rows // prefill_seq
+    ids = torch.randint(0, vocab, (prefill_rows,), generator=g).to(dev)
+    pos = torch.arange(prefill_seq, dtype=torch.int32).repeat(nseq).to(dev)
+    slots = torch.arange(nseq, dtype=torch.int32).repeat_interleave(prefill_seq).to(dev)
+    last = (torch.arange(1, nseq + 1, dtype=torch.int32) * prefill_seq - 1).to(dev)
+    for s in range(nseq):
+        model.kv.reserve(s, prefill_seq)
+    t = _time(lambda: model.forward(ids, pos, slots, (pos + 1).contiguous(), logit_rows=last, tokens_per_seq=[prefill_seq] * nseq), reps=3, warm=2)
+    prefill_tps = prefill_rows / t
+    for s in range(nseq):
+        model.kv.free(s)
+    fill(model)
+    dec = dec_cls(model, batch, use_graph=True)
+    dec.set_state(torch.randint(0, vocab, (batch,), generator=g).to(dev), [ctx] * batch, reserve_extra=steps + warmup + 2)
+    for _ in range(warmup):
+        dec.step()
+    torch.cuda.synchronize()
+    t0 = time.time()
+    for _ in range(steps):
+        dec.step()
+    torch.cuda.synchronize()
+    dt = (time.time() - t0) / steps
+    return prefill_tps, batch / dt, dt * 1e3
+
+
+def _kernels(sz, rows, batch, ctx, dev):
+    """Device time of single launches at the step's shapes: the design's kernels and the like kernels of the int8 decoder, each with the
+    share of its roofline (matrix products of `rows` rows: matrix-core peak; everything else: bytes moved / HBM rate)."""
+    from . import ops, ops_dense as D
+    W, ff, H, r, rd, vd = sz["width"], sz["ff"], sz["heads"], sz["kv_rank"], sz["rot_dim"], sz["vdim"]
+    Dc = r + rd
+    out = {}
+    g = torch.Generator(device=dev).manual_seed(1)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+
+    def row(name, t, flops=0.0, bytes_=0.0, peak=BF16_TFLOPS):
+        share = max(flops / t / (peak * 1e12), bytes_ / t / (HBM_GBS * 1e9))
+        out[name] = {"us": round(t * 1e6, 1), "roofline_share": round(share, 3)}
+
+    # ---- matrix products: the feed-forward's first product (gate and up, activation in the epilogue), prefill- and decode-sized ----
+    for n, tag in ((rows, "prefill"), (batch, "decode")):
+        a = rn(n, W)
+        w_gu = (rn(2 * ff, W) * 0.02).to(torch.bfloat16)
+        act = torch.empty(n, ff, device=dev)
+        t = _time(lambda: D.linear(a, w_gu, act, epilogue=D.EPI_GELU_MUL), 20)
+        row(f"linear_bf16_gate_up_{tag}", t, flops=2.0 * n * 2 * ff * W, bytes_=2.0 * 2 * ff * W + 4.0 * n * (W + ff))
+        a8 = torch.randint(-127, 127, (n, W), device=dev, dtype=torch.int8)
+        rs = torch.ones(n, device=dev)
+        w8 = torch.randint(-127, 127, (1, 2 * ff, W), device=dev, dtype=torch.int8)
+        ws = torch.ones(1, device=dev)
+        o8 = torch.empty(n, ff, device=dev)
+        t = _time(lambda: ops.gemm_i8(a8, rs, w8, ws, out=o8, epilogue=ops.EPI_SWIGLU), 20)
+        row(f"int8_decoder_gate_up_{tag}", t, flops=2.0 * n * 2 * ff * W, bytes_=1.0 * 2 * ff * W + 1.0 * n * W + 4.0 * n * ff, peak=I8_TOPS)
+    # ---- residual + norm ----
+    x, y, gp, b, nw = rn(rows, W), rn(rows, W), rn(rows, W), rn(W), rn(W)
+    o = torch.empty(rows, W, device=dev)
+    t = _time(lambda: D.gated_postnorm(x, nw, 2, 1e-6, alpha=1.0, y=y, gate_pre=gp, ldg=W, gate_bias=b, out=o), 20)
+    row("gated_postnorm_prefill", t, bytes_=4.0 * rows * W * 4)
+    st = ops.stats_alloc(4, dev)
+    t = _time(lambda: ops.fused_residual_norm(x, nw, 1e-6, add=y, h_out=x, normed=o, slot_base=0, stats=st), 20)
+    row("int8_decoder_residual_norm_prefill", t, bytes_=4.0 * rows * W * 4)
+    # ---- attention: a prompt's rows (sequences of 512 tokens), and one row per sequence at context ctx ----
+    for kind in ("prefill", "decode"):
+        if kind == "prefill":
+            seq = 512
+            n, nseq = rows, rows // seq
+            pos = torch.arange(seq, dtype=torch.int32).repeat(nseq).to(dev)
+            slots = torch.arange(nseq, dtype=torch.int32).repeat_interleave(seq).to(dev)
+            per_seq, keys = seq, seq * (seq + 1) / 2 * nseq
+        else:
+            n, nseq, per_seq = batch, batch, ctx
+            pos = torch.full((n,), ctx - 1, dtype=torch.int32, device=dev)
+            slots = torch.arange(n, dtype=torch.int32, device=dev)
+            keys = float(min(ctx, sz["window"])) * n
+        nb = (per_seq + 15) // 16
+        bt = torch.arange(nseq * nb, dtype=torch.int32, device=dev).view(nseq, nb).contiguous()
+        cache = (rn(nseq * nb, 16, Dc) * 0.5).to(torch.bfloat16)
+        q = rn(n, H, Dc) * 0.3
+        ol = torch.empty(n, H, r, device=dev)
+        t = _time(lambda: D.latent_attn(q, cache, bt, slots, pos, window=sz["window"], scale=0.1, heads=H, kv_rank=r, rot_dim=rd, out=ol), 5 if kind == "prefill" else 20)
+        row(f"latent_attn_{kind}", t, flops=2.0 * keys * H * (Dc + r), bytes_=(2.0 * keys * Dc if kind == "decode" else 0.0) + 4.0 * n * H * (Dc + r))
+        kvh, hd = sz["kv_heads"], W // H
+        kc = (rn(nseq * nb, 16, kvh, hd) * 0.5).to(torch.bfloat16)
+        vc = (rn(nseq * nb, 16, kvh, hd) * 0.5).to(torch.bfloat16)
+        q2 = rn(n, H, hd)
+        ctxl = (pos + 1).contiguous()
+        splits = 1 if kind == "prefill" else 8
+        ws = ops.attn_workspace(n, H, hd, splits, dev) if splits > 1 else None
+        o2 = torch.empty(n, H, hd, device=dev)
+        keys_full = keys if kind == "prefill" else float(ctx) * n
+        t = _time(lambda: ops.paged_attn(q2, kc, vc, bt, ctxl, slot_ids=slots, splits=splits, workspace=ws, out=o2), 5 if kind == "prefill" else 20)
+        row(f"int8_decoder_paged_attn_{kind}", t, flops=4.0 * keys_full * H * hd, bytes_=(4.0 * keys_full * kvh * hd if kind == "decode" else 0.0) + 8.0 * n * H * hd)
+    return out
+
+
+def run(args) -> dict:
+    from . import _lib, synth
+    from .config import ModelConfig
+    from .model import GreedyDecoder, I64MoEModel
+    from .morilorn import MorilornModel
+    _lib.load(), _lib.load_dense()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    batch, ctx, rows = args.batch, args.prompt_len, 4096
+    result = {"metric": "prefill / decode tokens/s of the Morilorn design beside the dense int8 decoder at equal sizes", "unit": "tokens/s", "n_gpus": 1,
+              "steps": args.steps, "warmup": args.warmup, "dtype": "bf16 matrix products, fp32 residual / norms / attention math (Morilorn); int8 dynamic Linears (closest model)",
+              "data": "synthetic", "config": {"batch": batch, "context": ctx, "prefill_step": f"{rows} rows = {rows // 512} prompts of 512 tokens"}, "sizes": {}}
+    for name in (args.design_sizes.split(",") if args.design_sizes else sorted(SIZES)):
+        sz = SIZES[name]
+        need_tokens = batch * (ctx + args.steps + args.warmup + 64)
+
+        def fill_latent(m):
+            g = torch.Generator(device=dev).manual_seed(5)
+            for t in m.kv.rows:
+                t.copy_((0.5 * torch.randn(t.shape, device=dev, generator=g)).to(t.dtype))
+
+        def fill_kv(m):
+            g = torch.Generator(device=dev).manual_seed(5)
+            for l in range(len(m.kv.k)):
+                m.kv.k[l].copy_(torch.randn(m.kv.k[l].shape, device=dev, generator=g).to(m.kv.k[l].dtype))
+                m.kv.v[l].copy_((0.6 * torch.randn(m.kv.v[l].shape, device=dev, generator=g)).to(m.kv.v[l].dtype))
+
+        cfg = synth.morilorn_config(width=sz["width"], layers=sz["layers"], heads=sz["heads"], dim=sz["dim"], rot_dim=sz["rot_dim"], vdim=sz["vdim"],
+                                    kv_rank=sz["kv_rank"], ff=sz["ff"], window=sz["window"])
+        model = MorilornModel(cfg, synth.make_morilorn_weights(cfg), device=dev, dtype="bfloat16", max_seqs=batch, num_kv_blocks=need_tokens // 16)
+        p, d, ms = _steps(model, GreedyDecoder, batch, ctx, rows, 512, args.steps, args.warmup, fill_latent, cfg.vocab, dev)
+        entry = {"morilorn": {"prefill_tokens_per_s": round(p, 1), "decode_tokens_per_s": round(d, 1), "decode_ms_per_step": round(ms, 3),
+                              "shape": {k: v for k, v in sz.items() if k != "kv_heads"}}}
+        del model
+        torch.cuda.empty_cache()
+        ccfg = ModelConfig(name=f"dense-{name}", hidden_size=sz["width"], num_layers=sz["layers"], num_heads=sz["width"] // 64, num_kv_heads=sz["kv_heads"],
+                           intermediate_size=sz["ff"], num_experts=1, shared_intermediate_size=0, top_k=1, primary_weight=1.0, table_routing=False,
+                           max_pos=(ctx + args.steps + args.warmup + 64 + 255) // 256 * 256)
+        cm = I64MoEModel(ccfg, synth.make_weights(ccfg, seed=0), device=dev, kv_dtype=torch.bfloat16, max_seqs=batch, num_kv_blocks=need_tokens // 16)
+        p, d, ms = _steps(cm, GreedyDecoder, batch, ctx, rows, 512, args.steps, args.warmup, fill_kv, ccfg.vocab_size, dev)
+        entry["int8_decoder"] = {"prefill_tokens_per_s": round(p, 1), "decode_tokens_per_s": round(d, 1), "decode_ms_per_step": round(ms, 3),
+                                 "shape": {"hidden": ccfg.hidden_size, "layers": ccfg.num_layers, "heads": ccfg.num_heads, "kv_heads": ccfg.num_kv_heads,
+                                           "intermediate": ccfg.intermediate_size}}
+        del cm
+        torch.cuda.empty_cache()
+        entry["kernels"] = _kernels(sz, rows, batch, ctx, dev)
+        result["sizes"][name] = entry
+    first = result["sizes"][sorted(result["sizes"])[0]]["morilorn"]
+    result["value"], result["ms_per_step"] = first["decode_tokens_per_s"], first["decode_ms_per_step"]
+    result["higher_is_better"], result["scaling"], result["vs_baseline"] = True, "weak", None
+    return result
+
+
+def main(args) -> int:
+    print(json.dumps(run(args)), flush=True)
+    return 0

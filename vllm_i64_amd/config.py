@@ -162,6 +162,11 @@ class MorilornConfig:
     def vocab_size(self) -> int:
         return self.vocab
 
+    @property
+    def max_pos(self) -> int:
+        """Positions are computed, not tabulated: a sequence is bounded by the page pool only."""
+        return 1 << 30
+
     @classmethod
     def from_dict(cls, d: dict) -> "MorilornConfig":
         norm = d.get("norm") or {}

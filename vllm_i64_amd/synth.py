@@ -76,3 +76,36 @@ def make_token_ids(cfg: ModelConfig, n: int, seed: int = 7, zipf: float = 0.0) -
     p = ranks.pow(-zipf)
     order = torch.randperm(cfg.vocab_size, generator=torch.Generator().manual_seed(99))
     return order[torch.multinomial(p / p.sum(), n, replacement=True, generator=g)]
+
+
+def morilorn_config(width: int = 1024, layers: int = 18, heads: int = 16, dim: int = 32, rot_dim: int = 32, vdim: int = 64, kv_rank: int = 256,
+                    ff: int = 4096, window: int = 1024, vocab: int = 32000, groups: int = 2):
+    """A Morilorn configuration with layers of a real model's proportions (random weights: make_morilorn_weights)."""
+    from .config import MorilornConfig
+    mixer = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "scale": (dim + rot_dim) ** -0.5,
+             "rot": {"base": 10000.0, "dims": rot_dim}, "mask": {"size": window}}
+    layer = {"type": "latent_attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}}
+    return MorilornConfig.from_dict({"architecture": "Morilorn", "vocab": vocab, "width": width, "layers": [layer] * layers, "embedding": {"scale": 1.0},
+                                     "postln_alpha": 1.0, "norm": {"eps": 1e-6, "groups": groups}, "logit_softcap": 30.0})
+
+
+def make_morilorn_weights(cfg, seed: int = 0, std: float = 0.02) -> Dict[str, torch.Tensor]:
+    """bf16 N(0, std) matrices, norm weights 1, gate biases 0, depth-mix weights 1 / (layers so far)."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg.width
+
+    def rn(*shape):
+        return torch.empty(*shape, dtype=torch.float32).normal_(0.0, std, generator=g).to(torch.bfloat16)
+
+    one = lambda n: torch.ones(n, dtype=torch.bfloat16)
+    w = {"embed": rn(cfg.vocab, W), "head": rn(cfg.vocab, W), "final.norm": one(W)}
+    for i, L in enumerate(cfg.layers):
+        p, m = f"l{i}.", L.mixer
+        w.update({p + "mix.q": rn(m.q_width, W), p + "mix.dkv": rn(m.cache_width, W), p + "mix.dkv.norm": one(m.kv_rank),
+                  p + "mix.uk": rn(m.heads * m.dim, m.kv_rank), p + "mix.uv": rn(m.heads * m.vdim, m.kv_rank), p + "mix.g": rn(m.heads * m.vdim, W),
+                  p + "mix.o": rn(W, m.heads * m.vdim), p + "rg1": rn(W, W), p + "rg1.b": torch.zeros(W, dtype=torch.bfloat16), p + "norm1": one(W),
+                  p + "dwa": torch.full((i + 2,), 1.0 / (i + 2), dtype=torch.bfloat16)})
+        if L.mlp is not None:
+            w.update({p + "mlp.gate": rn(L.mlp.ff, W), p + "mlp.up": rn(L.mlp.ff, W), p + "mlp.down": rn(W, L.mlp.ff), p + "rg2": rn(W, W),
+                      p + "rg2.b": torch.zeros(W, dtype=torch.bfloat16), p + "norm2": one(W)})
+    return w
