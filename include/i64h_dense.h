@@ -119,7 +119,10 @@ int i64h_latent_prep(const i64h_latent_prep_args* d, void* stream);
 /* i64h_latent_attn: row t (sequence slot_ids[t], position p = positions[t]) sees the cached rows j of its sequence with
  * 0 <= p - j < window (window <= 0: every j <= p);  s_j = scale * Q[t, h, :] . row_j;  ordinary softmax over the visible j;
  * out[t, h, :kv_rank] = sum_j w_j * row_j[:kv_rank].  Scores, weights and sums in fp32.  out fp32 [n, heads, kv_rank].
- * mode 0: picks the form by the launch (tile kernel for runs of rows of one sequence when the sizes fit it); 1: row form. */
+ * mode 1: one wave per (row, head), fp32 products, any sizes and cache type.  Modes 0 / 2 / 3 take the matrix-core form when the cache
+ * is bf16, kv_rank % 16 == 0 and <= 256, (kv_rank + rot_dim) % 8 == 0 and <= 320 (the row form otherwise): 2 (and 0) one wave per token
+ * and group of 16 heads (rows that are one per sequence), 3 one wave per 16 consecutive rows and head (portions of prompts; rows of
+ * different sequences in one tile are handled run by run). */
 typedef struct {
     const float* Q;
     const void* cache;

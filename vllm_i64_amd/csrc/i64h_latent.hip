@@ -5,7 +5,9 @@
 // q'_latent . latent_j + q_rot . key_rot_j and all heads read the same cached rows.
 //   latent_prep_kernel     : RMS norm of the latent, rotation of the shared key part and of every head's rotated query part,
 //                            cache write - one workgroup per token
-//   latent_attn_row_kernel : one wave per (token, head): 64 keys at a time, one key per lane for the scores (fp32 dot over the
+//   latent_attn_mfma_kernel: bf16 caches of aligned widths - 16 query vectors per wave (a token's heads, or a head's consecutive rows)
+//                            on the bf16 matrix cores, see below
+//   latent_attn_row_kernel : any width and cache type, true fp32 products: one wave per (token, head): 64 keys at a time, one key per lane for the scores (fp32 dot over the
 //                            cached row), online softmax over the wave, weighted row sum with the columns spread over the lanes
 #include "i64h_common.h"
 #include "i64h_dense.h"
@@ -145,6 +147,206 @@ __global__ __launch_bounds__(256) void latent_attn_row_kernel(const i64h_latent_
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------------
+// Matrix-core form (bf16 cache).  One wave per task of 16 query vectors that walk the same cached rows:
+//   head tiles: the (up to) 16 heads of a group of one token  - decode rows, one token per sequence;
+//   row tiles : 16 consecutive rows of the step for one head   - portions of prompts; rows of a tile that belong to different
+//               sequences are handled run by run (a run's keys are masked for every other row).
+// Per tile of 32 keys: scores S[16, 32] = Q K^T on v_mfma_f32_16x16x32_bf16 with the cached rows read straight from memory as B
+// fragments (8 consecutive values of one key per lane) and the scaled query carried as TWO bf16 terms (hi + lo, 16 mantissa bits),
+// masking and the online softmax in fp32 on the accumulator layout, the weights again as two bf16 terms through LDS into the
+// A layout, the tile's latent columns transposed through LDS (4 keys x 8 columns per lane and pass, 8-byte writes) into the B
+// layout of the second product, out[16, kv_rank] += P V in fp32.  Every product of two bf16 values is exact in fp32.
+#define LT_KD 10   // 32-wide steps over a cached row: kv_rank + rot_dim <= 320
+#define LT_NB 16   // 16-column blocks of the output: kv_rank <= 256
+#define LT_VLD 40  // halves per row of the transposed tile and of the weight planes (32 keys + 8: 16-byte aligned, conflict-poor)
+typedef __bf16 lt_v8bf __attribute__((ext_vector_type(8)));
+typedef float lt_v4f __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t lt_rne(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ void lt_split(float x, uint32_t& hi, uint32_t& lo) {
+    hi = lt_rne(x);
+    lo = lt_rne(x - __uint_as_float(hi << 16));
+}
+
+__global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_attn_args p, const int row_tiles) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x, n = lane & 15, kg = lane >> 4;
+    const int r = p.kv_rank, D = r + p.rot_dim, H = p.heads, bs = p.block_size, win = p.window;
+    uint16_t* Vt = (uint16_t*)smem;           // [r][LT_VLD]
+    uint16_t* Ph = Vt + r * LT_VLD;           // [16][LT_VLD]
+    uint16_t* Pl = Ph + 16 * LT_VLD;
+    int* info = (int*)(Pl + 16 * LT_VLD);     // [16] positions, [16] slots (-1: no such row)
+    const int64_t task = blockIdx.x;
+    const int64_t ntile = (p.n + 15) / 16;
+    const int hgroups = (H + 15) / 16;
+    auto row_of = [&](int m, int64_t& tok, int& head) -> bool {
+        if (row_tiles) {
+            tok = (task % ntile) * 16 + m;
+            head = (int)(task / ntile);
+            return tok < p.n;
+        }
+        tok = task / hgroups;
+        head = (int)(task % hgroups) * 16 + m;
+        return head < H;
+    };
+    int64_t tok_n;
+    int head_n;
+    const bool valid_n = row_of(n, tok_n, head_n);
+    if (lane < 16) {
+        info[lane] = valid_n ? p.positions[tok_n] : -1;
+        info[16 + lane] = valid_n ? p.slot_ids[tok_n] : -1;
+    }
+    // the scaled query of row n, columns ks * 32 + kg * 8 .. + 7, as two bf16 terms
+    uint4 Qh[LT_KD], Ql[LT_KD];
+    {
+        const float* q = p.Q + (tok_n * H + head_n) * D;
+#pragma unroll
+        for (int ks = 0; ks < LT_KD; ++ks) {
+            const int d0 = ks * 32 + kg * 8;
+            uint32_t h[8], l[8];
+            if (valid_n && d0 < D) {
+                const float4 a = *(const float4*)(q + d0), b = *(const float4*)(q + d0 + 4);
+                const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) lt_split(v[i] * p.scale, h[i], l[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = l[i] = 0;
+            }
+            Qh[ks] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+            Ql[ks] = make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16));
+        }
+    }
+    lt_v4f acc[LT_NB];
+#pragma unroll
+    for (int nb = 0; nb < LT_NB; ++nb) acc[nb] = lt_v4f{0, 0, 0, 0};
+    float mrow[4], lrow[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        mrow[g] = -INFINITY;
+        lrow[g] = 0.0f;
+    }
+    __syncthreads();
+    const uint16_t* cache = (const uint16_t*)p.cache;
+    int s0 = 0;
+    while (s0 < 16) {
+        const int sl = info[16 + s0];
+        if (sl < 0) {
+            ++s0;
+            continue;
+        }
+        int s1 = s0 + 1;
+        while (s1 < 16 && info[16 + s1] == sl) ++s1;
+        int lo = 0x7fffffff, hi = -1;
+        for (int i = s0; i < s1; ++i) {
+            const int pp = info[i];
+            hi = max(hi, pp);
+            lo = min(lo, win > 0 ? max(0, pp - win + 1) : 0);
+        }
+        const int32_t* bt = p.block_table + (int64_t)sl * p.max_blocks_per_seq;
+        for (int kb = lo & ~31; kb <= hi; kb += 32) {
+            lt_v4f S[2];
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                S[b] = lt_v4f{0, 0, 0, 0};
+                const int jc = min(kb + 16 * b + n, hi);
+                const uint16_t* rowp = cache + ((int64_t)bt[jc / bs] * bs + jc % bs) * D;
+#pragma unroll
+                for (int ks = 0; ks < LT_KD; ++ks) {
+                    if (ks * 32 < D) {
+                        const int d0 = ks * 32 + kg * 8;
+                        const uint4 kf = d0 < D ? *(const uint4*)(rowp + d0) : make_uint4(0, 0, 0, 0);
+                        S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Qh[ks]), __builtin_bit_cast(lt_v8bf, kf), S[b], 0, 0, 0);
+                        S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Ql[ks]), __builtin_bit_cast(lt_v8bf, kf), S[b], 0, 0, 0);
+                    }
+                }
+            }
+            float al[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int rr = kg * 4 + g;
+                const int pr = info[rr];
+                const bool in_run = rr >= s0 && rr < s1;
+                float sv[2];
+#pragma unroll
+                for (int b = 0; b < 2; ++b) {
+                    const int j = kb + 16 * b + n;
+                    const bool vis = in_run && j <= pr && (win <= 0 || pr - j < win);
+                    sv[b] = vis ? S[b][g] : -INFINITY;
+                }
+                const float mx = row16_max(fmaxf(sv[0], sv[1]));
+                const float mn = fmaxf(mrow[g], mx);
+                const float ms = mn == -INFINITY ? 0.0f : mn;
+                al[g] = expf(mrow[g] - ms);
+                const float p0 = expf(sv[0] - ms), p1 = expf(sv[1] - ms);
+                lrow[g] = lrow[g] * al[g] + group_sum(p0 + p1, 16);
+                mrow[g] = mn;
+                uint32_t h0, l0, h1, l1;
+                lt_split(p0, h0, l0);
+                lt_split(p1, h1, l1);
+                Ph[rr * LT_VLD + n] = (uint16_t)h0;
+                Pl[rr * LT_VLD + n] = (uint16_t)l0;
+                Ph[rr * LT_VLD + 16 + n] = (uint16_t)h1;
+                Pl[rr * LT_VLD + 16 + n] = (uint16_t)l1;
+            }
+            // the tile's latent columns, transposed: a lane takes 4 keys x 8 columns per pass
+            for (int idx = lane; idx < r; idx += 64) {     // 8 key groups x (r / 8) column groups = r blocks
+                const int kq = idx & 7, cg = idx >> 3;
+                uint4 w[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int jc = min(kb + kq * 4 + i, hi);
+                    w[i] = *(const uint4*)(cache + ((int64_t)bt[jc / bs] * bs + jc % bs) * D + cg * 8);
+                }
+                const uint32_t w0[4] = {w[0].x, w[0].y, w[0].z, w[0].w}, w1[4] = {w[1].x, w[1].y, w[1].z, w[1].w};
+                const uint32_t w2[4] = {w[2].x, w[2].y, w[2].z, w[2].w}, w3[4] = {w[3].x, w[3].y, w[3].z, w[3].w};
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const int q2 = c >> 1;
+                    uint32_t a, b;
+                    if (c & 1) {
+                        a = (w0[q2] >> 16) | (w1[q2] & 0xffff0000u);
+                        b = (w2[q2] >> 16) | (w3[q2] & 0xffff0000u);
+                    } else {
+                        a = (w0[q2] & 0xffffu) | (w1[q2] << 16);
+                        b = (w2[q2] & 0xffffu) | (w3[q2] << 16);
+                    }
+                    *(uint2*)&Vt[(cg * 8 + c) * LT_VLD + kq * 4] = make_uint2(a, b);
+                }
+            }
+            __syncthreads();
+            const uint4 pah = *(const uint4*)&Ph[n * LT_VLD + kg * 8], pal = *(const uint4*)&Pl[n * LT_VLD + kg * 8];
+#pragma unroll
+            for (int nb = 0; nb < LT_NB; ++nb) {
+                if (nb * 16 < r) {
+                    const uint4 vf = *(const uint4*)&Vt[(nb * 16 + n) * LT_VLD + kg * 8];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) acc[nb][g] *= al[g];
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, pah), __builtin_bit_cast(lt_v8bf, vf), acc[nb], 0, 0, 0);
+                    acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, pal), __builtin_bit_cast(lt_v8bf, vf), acc[nb], 0, 0, 0);
+                }
+            }
+            __syncthreads();
+        }
+        s0 = s1;
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        int64_t tok;
+        int head;
+        if (!row_of(kg * 4 + g, tok, head)) continue;
+        float* o = p.out + (tok * H + head) * r;
+        const float inv = 1.0f / lrow[g];
+#pragma unroll
+        for (int nb = 0; nb < LT_NB; ++nb)
+            if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g] * inv;
+    }
+}
+
 extern "C" {
 
 int i64h_latent_prep(const i64h_latent_prep_args* dp, void* stream) {
@@ -169,6 +371,17 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
     I64H_CHECK_ARG(d.Q && d.cache && d.block_table && d.slot_ids && d.positions && d.out, "latent_attn: null operand");
     if (d.n == 0) return 0;
     const int D = d.kv_rank + d.rot_dim;
+    const bool mfma_ok = d.cache_dtype == 2 && D % 8 == 0 && d.kv_rank % 16 == 0 && d.kv_rank <= 16 * LT_NB && D <= 32 * LT_KD &&
+                         (uintptr_t)d.Q % 16 == 0 && (uintptr_t)d.cache % 16 == 0;
+    if (d.mode != 1 && mfma_ok) {
+        const int row_tiles = d.mode == 3;
+        const int64_t tasks = row_tiles ? (d.n + 15) / 16 * d.heads : d.n * ((d.heads + 15) / 16);
+        I64H_CHECK_ARG(tasks < (1ll << 31), "latent_attn: too many tiles");
+        const size_t bytes = (size_t)d.kv_rank * LT_VLD * 2 + 2 * 16 * LT_VLD * 2 + 32 * 4;
+        hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks), dim3(64), bytes, (hipStream_t)stream, d, row_tiles);
+        I64H_CHECK_LAUNCH();
+        return 0;
+    }
     const size_t lds = (size_t)(4 * D + 512) * 4;
     I64H_CHECK_ARG(lds <= 64 * 1024, "latent_attn: cached rows of %d values do not fit", D);
     hipLaunchKernelGGL(latent_attn_row_kernel, dim3((unsigned)d.n, (unsigned)((d.heads + 3) / 4)), dim3(256), lds, (hipStream_t)stream, d);

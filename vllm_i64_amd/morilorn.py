@@ -23,6 +23,7 @@ import torch
 
 from . import ops_dense as D
 from .config import MorilornConfig
+from .model import attention_segments
 from .paged_cache import LatentCache
 
 
@@ -52,6 +53,7 @@ class _StepBuffers:
 
 class MorilornModel:
     MAX_BUFFER_SETS = int(os.environ.get("I64H_MAX_BUFFER_SETS", "8"))
+    ATTN_MAX_SEGMENTS = 4     # more runs than this in one step (finely interleaved kinds) collapse into one launch
 
     def __init__(self, cfg: MorilornConfig, weights: Dict[str, torch.Tensor], device="cuda:0", dtype: str = "bfloat16", max_seqs: int = 4,
                  num_kv_blocks: int = 256, kv_block: int = 16, cache_dtype: Optional[torch.dtype] = None):
@@ -128,7 +130,7 @@ class MorilornModel:
         """No launch of this runner waits on a grid barrier: nothing to read back."""
 
     # ---- mechanisms ----
-    def _mixer(self, B: _StepBuffers, d: dict, l: int, n: int, x: torch.Tensor, positions, slot_ids, kvc) -> None:
+    def _mixer(self, B: _StepBuffers, d: dict, l: int, n: int, x: torch.Tensor, positions, slot_ids, kvc, runs) -> None:
         """latent attention of layer l on the rows x; the result (before the output projection's gate of the residual) lands in B.y."""
         m, ex = d["m"], self.exact
         H, r, rd, D_ = m.heads, m.kv_rank, m.rot_dim, m.cache_width
@@ -142,7 +144,11 @@ class MorilornModel:
         # queries into latent space, per head: Q[:, h, :r] = q_unrotated[:, h, :] @ U_h
         D.linear(P, d["uk_t"], B.q, m=n, n=r, k=m.dim, a_off=d["q_off"], lda=N1, ldc=H * D_, batch=H, a_batch=m.dim + rd, w_batch=r * m.dim,
                  c_batch=D_, exact=ex)
-        D.latent_attn(B.q, cache, kvc.block_table, slot_ids, positions, window=m.window, scale=m.scale, heads=H, kv_rank=r, rot_dim=rd, out=B.olat, n=n)
+        # runs of rows that are one per sequence (decode rows: a wave takes a token's heads) and runs of prompt portions (a wave takes 16
+        # consecutive rows of one head), each one launch
+        for a, b, one_per_seq in runs:
+            D.latent_attn(B.q[a * H * D_: b * H * D_], cache, kvc.block_table, slot_ids[a:b], positions[a:b], window=m.window, scale=m.scale, heads=H,
+                          kv_rank=r, rot_dim=rd, out=B.olat[a * H * r: b * H * r], n=b - a, mode=2 if one_per_seq else 3)
         # summed latents into value space, per head, times the output gate sigmoid(W_g x)
         D.linear(B.olat, d["uv"], B.og, m=n, n=m.vdim, k=r, lda=H * r, ldc=H * m.vdim, batch=H, a_batch=r, w_batch=m.vdim * r, c_batch=m.vdim,
                  exact=ex, epilogue=D.EPI_MUL_SIGMOID, e=P, e_off=d["g_off"], lde=N1, e_batch=m.vdim)
@@ -156,7 +162,7 @@ class MorilornModel:
         the layer's window); logit_rows int32 [M] selects the rows whose logits are wanted (None = all).  Returns fp32 logits [M, V].
         record: dict filled with the stream after every layer ("l<i>.out": the mixed input of the next layer, "l<i>.x": the layer's own
         output).  kv: a LatentCache other than the runner's own.  ctx_len, max_ctx_hint, rows_are_slots and tokens_per_seq belong to
-        the shared step interface; this runner derives everything from positions."""
+        the shared step interface; tokens_per_seq (or rows_are_slots) only picks the attention launch forms."""
         cfg = self.cfg
         kvc = kv if kv is not None else self.kv
         n = token_ids.numel()
@@ -167,8 +173,12 @@ class MorilornModel:
         W, al, G, eps = cfg.width, cfg.postln_alpha, cfg.norm_groups, cfg.norm_eps
         D.embed_scaled(token_ids, self.embed, cfg.embedding_scale, B.hist[0])
         x = B.hist[0]
+        if tokens_per_seq is not None:
+            runs = attention_segments(tokens_per_seq, n, self.ATTN_MAX_SEGMENTS)
+        else:
+            runs = [(0, n, bool(rows_are_slots))]
         for l, d in enumerate(self.layers):
-            self._mixer(B, d, l, n, x, positions, slot_ids, kvc)
+            self._mixer(B, d, l, n, x, positions, slot_ids, kvc, runs)
             mixk = dict(hist=B.hist, hist_index=l + 1, mix_w=d["dwa"], mix_out=B.x)
             gate1 = dict(y=B.y, gate_pre=B.p, gate_off=d["rg_off"], ldg=d["n_in"], gate_bias=d["rg1_b"], alpha=al, n=n)
             if d["cfg"].mlp is None:
