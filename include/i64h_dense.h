@@ -137,7 +137,10 @@ typedef struct {
     int64_t n;
     int32_t heads, kv_rank, rot_dim;
     int32_t mode;
+    int32_t splits;      /* mode 2: every token's keys are dealt to this many waves (tiles of 32 keys in turn) and merged by a second launch */
+    float* workspace;    /* i64h_latent_attn_workspace_floats(n, heads, kv_rank, splits) floats when splits > 1 (NULL: no split) */
 } i64h_latent_attn_args;
+int64_t i64h_latent_attn_workspace_floats(int64_t n, int32_t heads, int32_t kv_rank, int32_t splits);
 int i64h_latent_attn(const i64h_latent_attn_args* d, void* stream);
 
 /* ---- sampling --------------------------------------------------------------------------------------------------------------

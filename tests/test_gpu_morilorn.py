@@ -82,7 +82,7 @@ SHAPES = {
 
 # ---- mechanisms alone ------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("exact", [False, True])
-@pytest.mark.parametrize("M,N,K", [(1, 5, 3), (7, 33, 20), (8, 72, 64), (70, 65, 100), (130, 200, 64), (3, 130, 256)])
+@pytest.mark.parametrize("M,N,K", [(1, 5, 3), (7, 33, 20), (8, 72, 64), (70, 65, 100), (130, 200, 64), (3, 130, 256), (64, 40, 168), (33, 16, 1024)])
 def test_linear_plain_and_epilogues(dev, exact, M, N, K):
     from vllm_i64_amd import ops_dense as D
     g = torch.Generator().manual_seed(M * 1000 + N + K)
@@ -92,7 +92,7 @@ def test_linear_plain_and_epilogues(dev, exact, M, N, K):
     ad, wd, ed = a.to(dev), w.to(dev), e.to(dev)
     A = a[:, 2:2 + K].double() if exact else bf16(a[:, 2:2 + K]).double()
     tol = 1e-5 if exact else 2e-5   # both forms sum exact products in fp32
-    for skinny in (1, 0):
+    for skinny in (3, 1, 0):     # rows <= 64 / rows <= 8 on their own kernels, then everything on the tile kernel
         D.call_dense("i64h_set_linear_skinny", skinny)
         out = torch.full((M, N + 4), 7.0, device=dev)
         D.linear(ad, wd, out, n=N, k=K, a_off=2, lda=K + 5, c_off=1, ldc=N + 4, exact=exact)
@@ -107,7 +107,7 @@ def test_linear_plain_and_epilogues(dev, exact, M, N, K):
         assert torch.allclose(out2.cpu().double(), ref * torch.sigmoid(e[:, 3:].double()), atol=1e-4, rtol=1e-4)
         D.linear(ad, wd, out2, n=N, k=K, a_off=2, lda=K + 5, exact=exact, epilogue=D.EPI_SOFTCAP, softcap=0.7)
         assert torch.allclose(out2.cpu().double(), 0.7 * torch.tanh(ref / 0.7), atol=1e-4, rtol=1e-4)
-    D.call_dense("i64h_set_linear_skinny", 1)
+    D.call_dense("i64h_set_linear_skinny", 3)
 
 
 @pytest.mark.parametrize("exact", [False, True])
@@ -258,6 +258,36 @@ def test_latent_attn_one_key_stands_out(dev, cache_dtype, window, r, e):
                 sees = p - star < window if window else True
                 close = torch.allclose(ref[i, 0], rows[star, :r].double(), atol=0.2)
                 assert close == sees, (window, star, p)
+
+
+def test_latent_attn_keys_dealt_to_several_waves(dev):
+    """Decode rows whose keys are split over waves and merged: same result as one wave per token, also when some shares are empty."""
+    from vllm_i64_amd import ops_dense as D
+    H, r, e = 5, 48, 16
+    g = torch.Generator().manual_seed(2)
+    lens = [1, 40, 333, 64]
+    nb = [(t + 15) // 16 for t in lens]
+    bt = torch.full((4, max(nb)), -1, dtype=torch.int32)
+    perm = torch.randperm(sum(nb), generator=g).to(torch.int32)
+    rows_of, at = [], 0
+    cache = torch.zeros(sum(nb), 16, r + e, dtype=torch.bfloat16, device=dev)
+    for s_, t in enumerate(lens):
+        bt[s_, :nb[s_]] = perm[at:at + nb[s_]]
+        rows = bf16(torch.randn(t, r + e, generator=g) * 0.7).float()
+        for b_i in range(nb[s_]):
+            part = rows[b_i * 16:(b_i + 1) * 16]
+            cache[int(perm[at + b_i]), :part.shape[0]] = part.to(dev).to(torch.bfloat16)
+        rows_of.append(rows.double())
+        at += nb[s_]
+    Q = torch.randn(4, H, r + e, generator=g)
+    pos = torch.tensor([t - 1 for t in lens], dtype=torch.int32)
+    for window in (0, 100):
+        ref = torch.cat([_ref_attn(Q[i:i + 1], rows_of[i], [lens[i] - 1], window, 0.4, r) for i in range(4)])
+        for splits in (1, 2, 5, 64):
+            out = torch.empty(4, H, r, device=dev)
+            D.latent_attn(Q.to(dev), cache, bt.to(dev), torch.arange(4, dtype=torch.int32, device=dev), pos.to(dev), window=window, scale=0.4, heads=H,
+                          kv_rank=r, rot_dim=e, out=out, mode=2, splits=splits)
+            assert torch.allclose(out.cpu().double(), ref, atol=1e-3, rtol=1e-3), (window, splits)
 
 
 def test_sample_rows(dev):

@@ -242,14 +242,14 @@ class LatentAttn(ctypes.Structure):
     """Mirror of i64h_latent_attn_args (include/i64h_dense.h)."""
     _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("slot_ids", _P), ("positions", _P), ("window", _I), ("scale", _F), ("out", _P), ("n", _L), ("heads", _I), ("kv_rank", _I),
-                ("rot_dim", _I), ("mode", _I)]
+                ("rot_dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P)]
 
 
 _dense: Optional[ctypes.CDLL] = None
 
 
 def dense_exported_symbols():
-    return ["i64h_last_error", "i64h_version", "i64h_device_check", *DENSE_SIGNATURES.keys()]
+    return ["i64h_last_error", "i64h_version", "i64h_device_check", "i64h_latent_attn_workspace_floats", *DENSE_SIGNATURES.keys()]
 
 
 def load_dense() -> ctypes.CDLL:
@@ -264,6 +264,8 @@ def load_dense() -> ctypes.CDLL:
     lib.i64h_last_error.restype = ctypes.c_char_p
     lib.i64h_last_error.argtypes = []
     lib.i64h_device_check.restype = _I
+    lib.i64h_latent_attn_workspace_floats.restype = _L
+    lib.i64h_latent_attn_workspace_floats.argtypes = [_L, _I, _I, _I]
     for name, sig in DENSE_SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = _I

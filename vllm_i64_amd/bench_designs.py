@@ -113,7 +113,11 @@ def _kernels(sz, rows, batch, ctx, dev):
         cache = (rn(nseq * nb, 16, Dc) * 0.5).to(torch.bfloat16)
         q = rn(n, H, Dc) * 0.3
         ol = torch.empty(n, H, r, device=dev)
-        t = _time(lambda: D.latent_attn(q, cache, bt, slots, pos, window=sz["window"], scale=0.1, heads=H, kv_rank=r, rot_dim=rd, out=ol), 5 if kind == "prefill" else 20)
+        # the launch forms the runner picks: a wave per 16 rows and head for prompts; a wave per token with the keys dealt to several waves for decode rows
+        sp = 1 if kind == "prefill" else max(1, min(1024 // max(1, n * ((H + 15) // 16)), int(keys / n) // 64, 64))
+        wsp = torch.empty(max(1, D.latent_attn_workspace_floats(n, H, r, sp)), device=dev) if sp > 1 else None
+        t = _time(lambda: D.latent_attn(q, cache, bt, slots, pos, window=sz["window"], scale=0.1, heads=H, kv_rank=r, rot_dim=rd, out=ol,
+                                        mode=3 if kind == "prefill" else 2, splits=sp, workspace=wsp), 5 if kind == "prefill" else 20)
         row(f"latent_attn_{kind}", t, flops=2.0 * keys * H * (Dc + r), bytes_=(2.0 * keys * Dc if kind == "decode" else 0.0) + 4.0 * n * H * (Dc + r))
         kvh, hd = sz["kv_heads"], W // H
         kc = (rn(nseq * nb, 16, kvh, hd) * 0.5).to(torch.bfloat16)

@@ -5,6 +5,8 @@
 //                          on two accumulators, * sigmoid(E), logit soft cap
 //   linear_skinny_kernel : the same product for at most I64H_SKINNY_ROWS rows (decode steps): the rows sit in LDS as bf16, every
 //                          wave streams four weight rows at a time with 16-byte loads and reduces over its lanes
+//   linear_rows64_kernel : at most 64 rows: 16 output columns per workgroup, the k steps dealt to its four waves, every operand read
+//                          from memory as a matrix-core fragment, partial tiles summed through LDS
 //   embed_scaled_kernel  : bf16 table row * scale -> fp32
 //   gated_postnorm_kernel: alpha * x + sigmoid(gate) * y -> RMS norm in groups -> (optional) weighted sum over the outputs of
 //                          all earlier layers; one workgroup per row, the row held in LDS between the passes
@@ -249,6 +251,82 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(const i64h_linear p,
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// At most 64 rows (decode steps, small batches), bf16 form.  A workgroup owns 16 output columns; its four waves take every fourth
+// 32-wide k step, each with up to four 16-row blocks of A against the one weight fragment, all operands read straight from memory
+// as matrix-core fragments (no staging, no barrier inside the loop); the four partial tiles meet in LDS, then the epilogue.
+// Many small workgroups fill the chip where a launch has few 64-column tiles, and the weights stream exactly once.
+template <int EPI>
+__global__ __launch_bounds__(256) void linear_rows64_kernel(const i64h_linear p) {
+    constexpr bool DUAL = EPI == I64H_EPI_GELU_MUL;
+    __shared__ float red[DUAL ? 2 : 1][4][64][17];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int n = lane & 15, kg = lane >> 4;
+    const int64_t b = blockIdx.z;
+    const int n0 = blockIdx.x * 16;
+    const int M = (int)p.M, N = p.N, K = p.K;
+    const int mblocks = (M + 15) / 16;
+    const bool cok = n0 + n < N;
+    const uint16_t* pw = (const uint16_t*)p.W + b * p.w_batch + (int64_t)(cok ? n0 + n : 0) * K;
+    const uint16_t* pw2 = pw + (int64_t)N * K;
+    const float* pa[4];
+    bool rok[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = i * 16 + n;
+        rok[i] = m < M;
+        const int64_t arow = rok[i] ? (p.a_rows ? (int64_t)p.a_rows[m] : m) : 0;
+        pa[i] = p.A + b * p.a_batch + arow * p.lda;
+    }
+    dn_v4f acc[4], acc2[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        acc[i] = dn_v4f{0, 0, 0, 0};
+        acc2[i] = dn_v4f{0, 0, 0, 0};
+    }
+    const int KT = (K + 31) / 32;
+    for (int kt = wv; kt < KT; kt += 4) {
+        const int k = kt * 32 + kg * 8;
+        const bool kin = k < K;
+        uint4 wf = make_uint4(0, 0, 0, 0), wf2 = make_uint4(0, 0, 0, 0);
+        if (cok && kin) {
+            wf = *(const uint4*)(pw + k);
+            if (DUAL) wf2 = *(const uint4*)(pw2 + k);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (i < mblocks) {
+                uint4 af = make_uint4(0, 0, 0, 0);
+                if (rok[i] && kin) {
+                    const float4 u = *(const float4*)(pa[i] + k), v = *(const float4*)(pa[i] + k + 4);
+                    af = make_uint4(dn_bf16_rne(u.x) | (dn_bf16_rne(u.y) << 16), dn_bf16_rne(u.z) | (dn_bf16_rne(u.w) << 16),
+                                    dn_bf16_rne(v.x) | (dn_bf16_rne(v.y) << 16), dn_bf16_rne(v.z) | (dn_bf16_rne(v.w) << 16));
+                }
+                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dn_v8bf, af), __builtin_bit_cast(dn_v8bf, wf), acc[i], 0, 0, 0);
+                if (DUAL) acc2[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dn_v8bf, af), __builtin_bit_cast(dn_v8bf, wf2), acc2[i], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            red[0][wv][i * 16 + kg * 4 + g][n] = acc[i][g];
+            if (DUAL) red[DUAL ? 1 : 0][wv][i * 16 + kg * 4 + g][n] = acc2[i][g];
+        }
+    __syncthreads();
+    float* C = p.C + b * p.c_batch;
+    for (int e = tid; e < 64 * 16; e += 256) {
+        const int m = e >> 4, c = e & 15;
+        if (m >= M || n0 + c >= N) continue;
+        const float s = ((red[0][0][m][c] + red[0][1][m][c]) + red[0][2][m][c]) + red[0][3][m][c];
+        float s2 = 0.0f;
+        if (DUAL) s2 = ((red[DUAL ? 1 : 0][0][m][c] + red[DUAL ? 1 : 0][1][m][c]) + red[DUAL ? 1 : 0][2][m][c]) + red[DUAL ? 1 : 0][3][m][c];
+        C[(int64_t)m * p.ldc + n0 + c] = dn_epilogue<EPI>(p, s, s2, b, m, n0 + c);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void embed_scaled_kernel(const int64_t* __restrict__ ids, const uint16_t* __restrict__ table, float scale,
                                                            float* __restrict__ out, int W, int64_t V) {
@@ -411,12 +489,15 @@ static void launch_tile(const i64h_linear& d, dim3 grid, hipStream_t s, int vecA
     }
 }
 
-static int g_skinny = 1;
+static int g_skinny = 1, g_rows64 = 1;
 
 extern "C" {
 
-int i64h_set_linear_skinny(int32_t on) {  // tuning / test knob: 0 = every launch on the tile kernel
-    g_skinny = on;
+// tuning / test knob, bit 0: launches of at most 8 rows on the weight-streaming kernel; bit 1: launches of at most 64 rows on the
+// fragment-streaming kernel (default 3: both; 0 = every launch on the tile kernel)
+int i64h_set_linear_skinny(int32_t on) {
+    g_skinny = on & 1;
+    g_rows64 = (on >> 1) & 1;
     return 0;
 }
 
@@ -444,6 +525,17 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
             case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), lds, s, d, cpb); break;
             default: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_STORE>), grid, dim3(256), lds, s, d, cpb); break;
+        }
+        I64H_CHECK_LAUNCH();
+        return 0;
+    }
+    if (g_rows64 && !d.exact && d.M <= 64 && vecA && vecW) {
+        const dim3 grid((unsigned)((d.N + 15) / 16), 1, (unsigned)d.batch);
+        switch (d.epilogue) {
+            case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_GELU_MUL>), grid, dim3(256), 0, s, d); break;
+            case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), 0, s, d); break;
+            case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d); break;
+            default: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_STORE>), grid, dim3(256), 0, s, d); break;
         }
         I64H_CHECK_LAUNCH();
         return 0;

@@ -172,15 +172,17 @@ __device__ __forceinline__ void lt_split(float x, uint32_t& hi, uint32_t& lo) {
     lo = lt_rne(x - __uint_as_float(hi << 16));
 }
 
-__global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_attn_args p, const int row_tiles) {
+__global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_attn_args p, const int row_tiles, const int splits) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x, n = lane & 15, kg = lane >> 4;
     const int r = p.kv_rank, D = r + p.rot_dim, H = p.heads, bs = p.block_size, win = p.window;
     uint16_t* Vt = (uint16_t*)smem;           // [r][LT_VLD]
     uint16_t* Ph = Vt + r * LT_VLD;           // [16][LT_VLD]
     uint16_t* Pl = Ph + 16 * LT_VLD;
-    int* info = (int*)(Pl + 16 * LT_VLD);     // [16] positions, [16] slots (-1: no such row)
+    int* info = (int*)(Pl + 16 * LT_VLD);     // [16] positions, [16] slots (-1: no such row), [32] cache rows of the tile's keys
+    int* rowoff = info + 32;
     const int64_t task = blockIdx.x;
+    const int split = blockIdx.y;
     const int64_t ntile = (p.n + 15) / 16;
     const int hgroups = (H + 15) / 16;
     auto row_of = [&](int m, int64_t& tok, int& head) -> bool {
@@ -200,10 +202,11 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
         info[lane] = valid_n ? p.positions[tok_n] : -1;
         info[16 + lane] = valid_n ? p.slot_ids[tok_n] : -1;
     }
-    // the scaled query of row n, columns ks * 32 + kg * 8 .. + 7, as two bf16 terms
+    // the query of row n times scale * log2(e) (the softmax runs on powers of two), columns ks * 32 + kg * 8 .. + 7, as two bf16 terms
     uint4 Qh[LT_KD], Ql[LT_KD];
     {
         const float* q = p.Q + (tok_n * H + head_n) * D;
+        const float qs = p.scale * 1.4426950408889634f;
 #pragma unroll
         for (int ks = 0; ks < LT_KD; ++ks) {
             const int d0 = ks * 32 + kg * 8;
@@ -212,7 +215,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
                 const float4 a = *(const float4*)(q + d0), b = *(const float4*)(q + d0 + 4);
                 const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
-                for (int i = 0; i < 8; ++i) lt_split(v[i] * p.scale, h[i], l[i]);
+                for (int i = 0; i < 8; ++i) lt_split(v[i] * qs, h[i], l[i]);
             } else {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) h[i] = l[i] = 0;
@@ -248,13 +251,17 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
             lo = min(lo, win > 0 ? max(0, pp - win + 1) : 0);
         }
         const int32_t* bt = p.block_table + (int64_t)sl * p.max_blocks_per_seq;
-        for (int kb = lo & ~31; kb <= hi; kb += 32) {
+        for (int kb = (lo & ~31) + 32 * split; kb <= hi; kb += 32 * splits) {
+            if (lane < 32) {
+                const int jc = min(kb + lane, hi);
+                rowoff[lane] = bt[jc / bs] * bs + jc % bs;
+            }
+            __syncthreads();
             lt_v4f S[2];
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 S[b] = lt_v4f{0, 0, 0, 0};
-                const int jc = min(kb + 16 * b + n, hi);
-                const uint16_t* rowp = cache + ((int64_t)bt[jc / bs] * bs + jc % bs) * D;
+                const uint16_t* rowp = cache + (int64_t)rowoff[16 * b + n] * D;
 #pragma unroll
                 for (int ks = 0; ks < LT_KD; ++ks) {
                     if (ks * 32 < D) {
@@ -262,6 +269,11 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
                         const uint4 kf = d0 < D ? *(const uint4*)(rowp + d0) : make_uint4(0, 0, 0, 0);
                         S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Qh[ks]), __builtin_bit_cast(lt_v8bf, kf), S[b], 0, 0, 0);
                         S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Ql[ks]), __builtin_bit_cast(lt_v8bf, kf), S[b], 0, 0, 0);
+                        if (d0 < r) {   // the same registers, transposed, are the second product's operand: column d0 + c of key 16 b + n
+                            const uint32_t kw[4] = {kf.x, kf.y, kf.z, kf.w};
+#pragma unroll
+                            for (int c = 0; c < 8; ++c) Vt[(d0 + c) * LT_VLD + 16 * b + n] = (uint16_t)(kw[c >> 1] >> (16 * (c & 1)));
+                        }
                     }
                 }
             }
@@ -281,8 +293,8 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
                 const float mx = row16_max(fmaxf(sv[0], sv[1]));
                 const float mn = fmaxf(mrow[g], mx);
                 const float ms = mn == -INFINITY ? 0.0f : mn;
-                al[g] = expf(mrow[g] - ms);
-                const float p0 = expf(sv[0] - ms), p1 = expf(sv[1] - ms);
+                al[g] = __builtin_amdgcn_exp2f(mrow[g] - ms);
+                const float p0 = __builtin_amdgcn_exp2f(sv[0] - ms), p1 = __builtin_amdgcn_exp2f(sv[1] - ms);
                 lrow[g] = lrow[g] * al[g] + group_sum(p0 + p1, 16);
                 mrow[g] = mn;
                 uint32_t h0, l0, h1, l1;
@@ -292,31 +304,6 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
                 Pl[rr * LT_VLD + n] = (uint16_t)l0;
                 Ph[rr * LT_VLD + 16 + n] = (uint16_t)h1;
                 Pl[rr * LT_VLD + 16 + n] = (uint16_t)l1;
-            }
-            // the tile's latent columns, transposed: a lane takes 4 keys x 8 columns per pass
-            for (int idx = lane; idx < r; idx += 64) {     // 8 key groups x (r / 8) column groups = r blocks
-                const int kq = idx & 7, cg = idx >> 3;
-                uint4 w[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int jc = min(kb + kq * 4 + i, hi);
-                    w[i] = *(const uint4*)(cache + ((int64_t)bt[jc / bs] * bs + jc % bs) * D + cg * 8);
-                }
-                const uint32_t w0[4] = {w[0].x, w[0].y, w[0].z, w[0].w}, w1[4] = {w[1].x, w[1].y, w[1].z, w[1].w};
-                const uint32_t w2[4] = {w[2].x, w[2].y, w[2].z, w[2].w}, w3[4] = {w[3].x, w[3].y, w[3].z, w[3].w};
-#pragma unroll
-                for (int c = 0; c < 8; ++c) {
-                    const int q2 = c >> 1;
-                    uint32_t a, b;
-                    if (c & 1) {
-                        a = (w0[q2] >> 16) | (w1[q2] & 0xffff0000u);
-                        b = (w2[q2] >> 16) | (w3[q2] & 0xffff0000u);
-                    } else {
-                        a = (w0[q2] & 0xffffu) | (w1[q2] << 16);
-                        b = (w2[q2] & 0xffffu) | (w3[q2] << 16);
-                    }
-                    *(uint2*)&Vt[(cg * 8 + c) * LT_VLD + kq * 4] = make_uint2(a, b);
-                }
             }
             __syncthreads();
             const uint4 pah = *(const uint4*)&Ph[n * LT_VLD + kg * 8], pal = *(const uint4*)&Pl[n * LT_VLD + kg * 8];
@@ -334,6 +321,22 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
         }
         s0 = s1;
     }
+    if (splits > 1) {
+        // partial result of this share of the keys: [16 rows][kv_rank unnormalised sums | maximum (log2 units) | sum of weights]
+        float* w = p.workspace + ((int64_t)task * splits + split) * 16 * (r + 2);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float* o = w + (kg * 4 + g) * (r + 2);
+#pragma unroll
+            for (int nb = 0; nb < LT_NB; ++nb)
+                if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g];
+            if (n == 0) {
+                o[r] = mrow[g];
+                o[r + 1] = lrow[g];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         int64_t tok;
@@ -344,6 +347,34 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
 #pragma unroll
         for (int nb = 0; nb < LT_NB; ++nb)
             if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g] * inv;
+    }
+}
+
+// the shares of a token's keys, merged: one workgroup per (token, group of 16 heads), a wave per head at a time; lane s holds share s's
+// maximum and weight sum (at most 64 shares), every lane then sums its columns over the shares
+__global__ __launch_bounds__(256) void latent_attn_merge_kernel(const i64h_latent_attn_args p, const int splits) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int r = p.kv_rank, H = p.heads;
+    const int hgroups = (H + 15) / 16;
+    const int64_t task = blockIdx.x, tok = task / hgroups;
+    const float* w = p.workspace + task * splits * 16 * (r + 2);
+    for (int m = wv; m < 16; m += 4) {
+        const int head = (int)(task % hgroups) * 16 + m;
+        if (head >= H) continue;
+        const float* mine = w + ((int64_t)min(lane, splits - 1) * 16 + m) * (r + 2);
+        const float ms = lane < splits ? mine[r] : -INFINITY, ls = lane < splits ? mine[r + 1] : 0.0f;
+        const float mx = wave_max(ms);
+        const float f = __builtin_amdgcn_exp2f(ms - mx);      // share `lane`'s factor (0 for an empty share)
+        const float den = wave_sum(f * ls);
+        for (int c0 = 0; c0 < r; c0 += 64) {
+            const int c = c0 + lane;
+            float num = 0.0f;
+            for (int s = 0; s < splits; ++s) {
+                const float fs = __shfl(f, s);
+                if (c < r) num += fs * w[((int64_t)s * 16 + m) * (r + 2) + c];
+            }
+            if (c < r) p.out[(tok * H + head) * r + c] = num / den;
+        }
     }
 }
 
@@ -362,6 +393,11 @@ int i64h_latent_prep(const i64h_latent_prep_args* dp, void* stream) {
     return 0;
 }
 
+int64_t i64h_latent_attn_workspace_floats(int64_t n, int32_t heads, int32_t kv_rank, int32_t splits) {
+    if (splits <= 1) return 0;
+    return n * ((heads + 15) / 16) * (int64_t)(splits > 64 ? 64 : splits) * 16 * (kv_rank + 2);
+}
+
 int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
     I64H_CHECK_ARG(dp != nullptr, "latent_attn: no descriptor");
     const i64h_latent_attn_args& d = *dp;
@@ -377,9 +413,14 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
         const int row_tiles = d.mode == 3;
         const int64_t tasks = row_tiles ? (d.n + 15) / 16 * d.heads : d.n * ((d.heads + 15) / 16);
         I64H_CHECK_ARG(tasks < (1ll << 31), "latent_attn: too many tiles");
-        const size_t bytes = (size_t)d.kv_rank * LT_VLD * 2 + 2 * 16 * LT_VLD * 2 + 32 * 4;
-        hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks), dim3(64), bytes, (hipStream_t)stream, d, row_tiles);
+        const int splits = (!row_tiles && d.workspace && d.splits > 1) ? (d.splits > 64 ? 64 : d.splits) : 1;
+        const size_t bytes = (size_t)d.kv_rank * LT_VLD * 2 + 2 * 16 * LT_VLD * 2 + 64 * 4;
+        hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, row_tiles, splits);
         I64H_CHECK_LAUNCH();
+        if (splits > 1) {
+            hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tasks), dim3(256), 0, (hipStream_t)stream, d, splits);
+            I64H_CHECK_LAUNCH();
+        }
         return 0;
     }
     const size_t lds = (size_t)(4 * D + 512) * 4;

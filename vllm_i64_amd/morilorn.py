@@ -49,11 +49,13 @@ class _StepBuffers:
         self.act = torch.empty(n * max(model.max_ff, 1), **f32)
         self.xf = torch.empty(m, W, **f32)
         self.logits = torch.empty(m, model.cfg.vocab, **f32)
+        self.attn_ws: Dict[tuple, torch.Tensor] = {}   # partial results of split attention launches by (rows, heads, rank, splits)
 
 
 class MorilornModel:
     MAX_BUFFER_SETS = int(os.environ.get("I64H_MAX_BUFFER_SETS", "8"))
     ATTN_MAX_SEGMENTS = 4     # more runs than this in one step (finely interleaved kinds) collapse into one launch
+    ATTN_WAVES = 1024         # waves a decode-sized attention launch aims at (256 CUs, four SIMDs each)
 
     def __init__(self, cfg: MorilornConfig, weights: Dict[str, torch.Tensor], device="cuda:0", dtype: str = "bfloat16", max_seqs: int = 4,
                  num_kv_blocks: int = 256, kv_block: int = 16, cache_dtype: Optional[torch.dtype] = None):
@@ -130,7 +132,7 @@ class MorilornModel:
         """No launch of this runner waits on a grid barrier: nothing to read back."""
 
     # ---- mechanisms ----
-    def _mixer(self, B: _StepBuffers, d: dict, l: int, n: int, x: torch.Tensor, positions, slot_ids, kvc, runs) -> None:
+    def _mixer(self, B: _StepBuffers, d: dict, l: int, n: int, x: torch.Tensor, positions, slot_ids, kvc, runs, ctx_hint: int) -> None:
         """latent attention of layer l on the rows x; the result (before the output projection's gate of the residual) lands in B.y."""
         m, ex = d["m"], self.exact
         H, r, rd, D_ = m.heads, m.kv_rank, m.rot_dim, m.cache_width
@@ -147,8 +149,19 @@ class MorilornModel:
         # runs of rows that are one per sequence (decode rows: a wave takes a token's heads) and runs of prompt portions (a wave takes 16
         # consecutive rows of one head), each one launch
         for a, b, one_per_seq in runs:
+            splits, ws = 1, None
+            if one_per_seq:
+                # few rows with long contexts: a token's keys are dealt to several waves, about four waves per CU in the launch, a wave
+                # keeping at least two tiles of 32 keys
+                keys = min(m.window, ctx_hint) if m.window > 0 else ctx_hint
+                splits = max(1, min(self.ATTN_WAVES // max(1, (b - a) * ((H + 15) // 16)), keys // 64, 64))
+                if splits > 1:
+                    key = (b - a, H, r, splits)
+                    ws = B.attn_ws.get(key)
+                    if ws is None:
+                        ws = B.attn_ws[key] = torch.empty(max(1, D.latent_attn_workspace_floats(b - a, H, r, splits)), dtype=torch.float32, device=self.device)
             D.latent_attn(B.q[a * H * D_: b * H * D_], cache, kvc.block_table, slot_ids[a:b], positions[a:b], window=m.window, scale=m.scale, heads=H,
-                          kv_rank=r, rot_dim=rd, out=B.olat[a * H * r: b * H * r], n=b - a, mode=2 if one_per_seq else 3)
+                          kv_rank=r, rot_dim=rd, out=B.olat[a * H * r: b * H * r], n=b - a, mode=2 if one_per_seq else 3, splits=splits, workspace=ws)
         # summed latents into value space, per head, times the output gate sigmoid(W_g x)
         D.linear(B.olat, d["uv"], B.og, m=n, n=m.vdim, k=r, lda=H * r, ldc=H * m.vdim, batch=H, a_batch=r, w_batch=m.vdim * r, c_batch=m.vdim,
                  exact=ex, epilogue=D.EPI_MUL_SIGMOID, e=P, e_off=d["g_off"], lde=N1, e_batch=m.vdim)
@@ -178,7 +191,7 @@ class MorilornModel:
         else:
             runs = [(0, n, bool(rows_are_slots))]
         for l, d in enumerate(self.layers):
-            self._mixer(B, d, l, n, x, positions, slot_ids, kvc, runs)
+            self._mixer(B, d, l, n, x, positions, slot_ids, kvc, runs, int(max_ctx_hint))
             mixk = dict(hist=B.hist, hist_index=l + 1, mix_w=d["dwa"], mix_out=B.x)
             gate1 = dict(y=B.y, gate_pre=B.p, gate_off=d["rg_off"], ldg=d["n_in"], gate_bias=d["rg1_b"], alpha=al, n=n)
             if d["cfg"].mlp is None:

@@ -107,18 +107,30 @@ def latent_prep(p: torch.Tensor, *, q_off: int, dkv_off: int, heads: int, dim: i
 
 def latent_attn(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, slot_ids: torch.Tensor, positions: torch.Tensor, *,
                 window: int, scale: float, heads: int, kv_rank: int, rot_dim: int, out: torch.Tensor, n: Optional[int] = None,
-                mode: int = 0) -> torch.Tensor:
+                mode: int = 0, splits: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     _chk(q, torch.float32, "q"), _chk(out, torch.float32, "out"), _chk(cache, None, "cache")
     _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids"), _chk(block_table, torch.int32, "block_table")
     rows = int(n if n is not None else positions.numel())
     D = kv_rank + rot_dim
     if cache.shape[-1] != D or q.numel() < rows * heads * D or out.numel() < rows * heads * kv_rank:
         raise _lib.I64HError("latent_attn: cache / query / output shapes do not fit the sizes")
+    if splits > 1:
+        need = latent_attn_workspace_floats(rows, heads, kv_rank, splits)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.float32, device=q.device)
+        _chk(workspace, torch.float32, "workspace")
+        if workspace.numel() < need:
+            raise _lib.I64HError(f"latent_attn: workspace of {workspace.numel()} floats, {need} needed")
     d = _lib.LatentAttn(Q=ptr(q), cache=ptr(cache), cache_dtype=CACHE_DTYPE_CODE[cache.dtype], block_table=ptr(block_table),
                         max_blocks_per_seq=block_table.shape[1], block_size=cache.shape[-2], slot_ids=ptr(slot_ids), positions=ptr(positions),
-                        window=int(window), scale=float(scale), out=ptr(out), n=rows, heads=heads, kv_rank=kv_rank, rot_dim=rot_dim, mode=mode)
+                        window=int(window), scale=float(scale), out=ptr(out), n=rows, heads=heads, kv_rank=kv_rank, rot_dim=rot_dim, mode=mode,
+                        splits=int(splits) if splits > 1 else 1, workspace=ptr(workspace) if splits > 1 else 0)
     call_dense("i64h_latent_attn", _ref(d), _stream())
     return out
+
+
+def latent_attn_workspace_floats(n: int, heads: int, kv_rank: int, splits: int) -> int:
+    return int(_lib.load_dense().i64h_latent_attn_workspace_floats(n, heads, kv_rank, splits))
 
 
 def sample_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None, temperature: Optional[torch.Tensor] = None,
