@@ -350,31 +350,36 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
     }
 }
 
-// the shares of a token's keys, merged: one workgroup per (token, group of 16 heads), a wave per head at a time; lane s holds share s's
-// maximum and weight sum (at most 64 shares), every lane then sums its columns over the shares
-__global__ __launch_bounds__(256) void latent_attn_merge_kernel(const i64h_latent_attn_args p, const int splits) {
-    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+// the shares of a token's keys, merged: one wave per (token, head); lane s holds share s's maximum and weight sum (at most 64
+// shares), then every lane sums its columns over the shares, eight loads in flight at a time
+__global__ __launch_bounds__(64) void latent_attn_merge_kernel(const i64h_latent_attn_args p, const int splits) {
+    __shared__ float sf[64];
+    const int lane = threadIdx.x;
     const int r = p.kv_rank, H = p.heads;
     const int hgroups = (H + 15) / 16;
     const int64_t task = blockIdx.x, tok = task / hgroups;
-    const float* w = p.workspace + task * splits * 16 * (r + 2);
-    for (int m = wv; m < 16; m += 4) {
-        const int head = (int)(task % hgroups) * 16 + m;
-        if (head >= H) continue;
-        const float* mine = w + ((int64_t)min(lane, splits - 1) * 16 + m) * (r + 2);
-        const float ms = lane < splits ? mine[r] : -INFINITY, ls = lane < splits ? mine[r + 1] : 0.0f;
-        const float mx = wave_max(ms);
-        const float f = __builtin_amdgcn_exp2f(ms - mx);      // share `lane`'s factor (0 for an empty share)
-        const float den = wave_sum(f * ls);
-        for (int c0 = 0; c0 < r; c0 += 64) {
-            const int c = c0 + lane;
-            float num = 0.0f;
-            for (int s = 0; s < splits; ++s) {
-                const float fs = __shfl(f, s);
-                if (c < r) num += fs * w[((int64_t)s * 16 + m) * (r + 2) + c];
-            }
-            if (c < r) p.out[(tok * H + head) * r + c] = num / den;
+    const int m = blockIdx.y;
+    const int head = (int)(task % hgroups) * 16 + m;
+    if (head >= H) return;
+    const float* w = p.workspace + (task * splits * 16 + m) * (r + 2);      // share s: + s * 16 * (r + 2)
+    const int64_t stride = (int64_t)16 * (r + 2);
+    const float* mine = w + (int64_t)min(lane, splits - 1) * stride;
+    const float ms = lane < splits ? mine[r] : -INFINITY, ls = lane < splits ? mine[r + 1] : 0.0f;
+    const float mx = wave_max(ms);
+    const float f = __builtin_amdgcn_exp2f(ms - mx);      // share `lane`'s factor (0 for an empty share)
+    const float den = wave_sum(f * ls);
+    sf[lane] = lane < splits ? f : 0.0f;
+    __syncthreads();
+    for (int c = lane; c < r; c += 64) {
+        float num = 0.0f;
+        for (int s0 = 0; s0 < splits; s0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = s0 + u < splits ? w[(int64_t)(s0 + u) * stride + c] : 0.0f;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) num += sf[(s0 + u) & 63] * v[u];
         }
+        p.out[(tok * H + head) * r + c] = num / den;
     }
 }
 
@@ -418,7 +423,7 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
         hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, row_tiles, splits);
         I64H_CHECK_LAUNCH();
         if (splits > 1) {
-            hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tasks), dim3(256), 0, (hipStream_t)stream, d, splits);
+            hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tasks, 16), dim3(64), 0, (hipStream_t)stream, d, splits);
             I64H_CHECK_LAUNCH();
         }
         return 0;
