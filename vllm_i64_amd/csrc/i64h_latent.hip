@@ -172,7 +172,7 @@ __device__ __forceinline__ void lt_split(float x, uint32_t& hi, uint32_t& lo) {
     lo = lt_rne(x - __uint_as_float(hi << 16));
 }
 
-__global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_attn_args p, const int row_tiles, const int splits) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void latent_attn_mfma_kernel(const i64h_latent_attn_args p, const int row_tiles, const int splits) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x, n = lane & 15, kg = lane >> 4;
     const int r = p.kv_rank, D = r + p.rot_dim, H = p.heads, bs = p.block_size, win = p.window;
@@ -183,12 +183,11 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_kernel(const i64h_latent_
     int* rowoff = info + 32;
     const int64_t task = blockIdx.x;
     const int split = blockIdx.y;
-    const int64_t ntile = (p.n + 15) / 16;
     const int hgroups = (H + 15) / 16;
     auto row_of = [&](int m, int64_t& tok, int& head) -> bool {
-        if (row_tiles) {
-            tok = (task % ntile) * 16 + m;
-            head = (int)(task / ntile);
+        if (row_tiles) {     // the heads of a row tile are neighbours in the launch: they walk the same cached rows at the same time
+            tok = (task / H) * 16 + m;
+            head = (int)(task % H);
             return tok < p.n;
         }
         tok = task / hgroups;
