@@ -92,7 +92,7 @@ def test_linear_plain_and_epilogues(dev, exact, M, N, K):
     ad, wd, ed = a.to(dev), w.to(dev), e.to(dev)
     A = a[:, 2:2 + K].double() if exact else bf16(a[:, 2:2 + K]).double()
     tol = 1e-5 if exact else 2e-5   # both forms sum exact products in fp32
-    for skinny in (3, 1, 0):     # rows <= 64 / rows <= 8 on their own kernels, then everything on the tile kernel
+    for skinny in (7, 1, 0):     # every kernel where it applies; rows <= 8 on their own kernel only; everything on the 64 x 64 tile kernel
         D.call_dense("i64h_set_linear_skinny", skinny)
         out = torch.full((M, N + 4), 7.0, device=dev)
         D.linear(ad, wd, out, n=N, k=K, a_off=2, lda=K + 5, c_off=1, ldc=N + 4, exact=exact)
@@ -155,6 +155,33 @@ def test_gated_postnorm_and_depth_mix(dev, W, groups):
     out2 = torch.empty(2, W, device=dev)
     D.gated_postnorm(x.to(dev), nw.to(dev), groups, 1e-3, x_rows=rows.to(dev), out=out2)
     assert torch.allclose(out2.cpu().double(), R.rms_norm(x[rows.long()].double(), nw.double(), 1e-3, groups), atol=2e-6, rtol=2e-6)
+
+
+@pytest.mark.parametrize("epilogue", [0, 1, 2, 3])
+def test_linear_large_tiles(dev, epilogue):
+    """A launch with enough 128 x 128 tiles for the large-tile kernel, edges in M, N and K, against the 64 x 64 kernel's result."""
+    from vllm_i64_amd import ops_dense as D
+    g = torch.Generator().manual_seed(epilogue)
+    M, N, K = 2000, 2100, 104
+    a = torch.randn(M, K, generator=g).to(dev)
+    w = bf16(torch.randn(2 * N, K, generator=g) / math.sqrt(K)).to(dev)
+    e = torch.randn(M, N, generator=g).to(dev)
+    outs = []
+    for knob in (7, 0):
+        D.call_dense("i64h_set_linear_skinny", knob)
+        out = torch.empty(M, N, device=dev)
+        D.linear(a, w, out, n=N, k=K, epilogue=epilogue, e=e if epilogue == 2 else None, lde=N, softcap=1.3 if epilogue == 3 else 0.0)
+        outs.append(out.cpu())
+    D.call_dense("i64h_set_linear_skinny", 3)
+    assert torch.equal(outs[0], outs[1])       # the same products summed in the same order
+    ref = bf16(a.cpu()).double() @ w.cpu()[:N].double().T
+    if epilogue == 1:
+        ref = R.gelu_tanh(ref) * (bf16(a.cpu()).double() @ w.cpu()[N:].double().T)
+    elif epilogue == 2:
+        ref = ref * torch.sigmoid(e.cpu().double())
+    elif epilogue == 3:
+        ref = 1.3 * torch.tanh(ref / 1.3)
+    assert torch.allclose(outs[0].double(), ref, atol=1e-4, rtol=1e-4)
 
 
 def test_embed_scaled(dev):

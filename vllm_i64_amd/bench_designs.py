@@ -12,7 +12,7 @@ HBM_GBS, BF16_TFLOPS, I8_TOPS = 8000.0, 2500.0, 5000.0      # MI355X: HBM3E, den
 
 SIZES = {
     "w1024": dict(width=1024, layers=18, heads=16, dim=32, rot_dim=32, vdim=64, kv_rank=256, ff=4096, window=1024, kv_heads=4),
-    "w2048": dict(width=2048, layers=8, heads=32, dim=32, rot_dim=32, vdim=64, kv_rank=512, ff=8192, window=1024, kv_heads=8),
+    "w2048": dict(width=2048, layers=8, heads=32, dim=64, rot_dim=32, vdim=64, kv_rank=256, ff=8192, window=1024, kv_heads=8),
 }
 
 

@@ -3,6 +3,7 @@
 //                          bf16 while staged) or v_mfma_f32_16x16x4_f32 (W widened while staged: true 32-bit); batched over
 //                          blockIdx.z (per-head weights on column blocks of wider matrices); epilogues: gelu_tanh(gate) * up
 //                          on two accumulators, * sigmoid(E), logit soft cap
+//   linear_tile128_kernel: bf16 form, 128 x 128 tiles (waves of 64 x 64); behind a knob, measured slower at the sizes tried
 //   linear_skinny_kernel : the same product for at most I64H_SKINNY_ROWS rows (decode steps): the rows sit in LDS as bf16, every
 //                          wave streams four weight rows at a time with 16-byte loads and reduces over its lanes
 //   linear_rows64_kernel : at most 64 rows: 16 output columns per workgroup, the k steps dealt to its four waves, every operand read
@@ -166,6 +167,127 @@ __global__ __launch_bounds__(256) void linear_tile_kernel(const i64h_linear p, c
             for (int j = 0; j < 2; ++j) {
                 const int c = n0 + wn * 32 + j * 16 + fr;
                 if (c < N) C[r * p.ldc + c] = dn_epilogue<EPI>(p, acc[i][j][reg], acc2[i][j][reg], b, r, c);
+            }
+        }
+}
+
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// The bf16 form for launches with many tiles: 128 x 128 per workgroup, four waves of 64 x 64 (16 matrix instructions per wave and
+// 32-wide k step against 8 fragment reads - four times the 64 x 64 kernel's ratio), the same staging scheme.
+template <int EPI>
+__global__ __launch_bounds__(256) void linear_tile128_kernel(const i64h_linear p, const int vecA, const int vecW) {
+    constexpr bool DUAL = EPI == I64H_EPI_GELU_MUL;
+    constexpr int LD = 40;
+    __shared__ __attribute__((aligned(16))) uint16_t sA[2][128][LD];
+    __shared__ __attribute__((aligned(16))) uint16_t sB[2][128][LD];
+    __shared__ __attribute__((aligned(16))) uint16_t sB2[DUAL ? 2 : 1][DUAL ? 128 : 1][LD];
+    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+    const int wm = wid >> 1, wn = wid & 1;
+    const int64_t b = blockIdx.z;
+    const int64_t m0 = (int64_t)blockIdx.y * 128;
+    const int n0 = blockIdx.x * 128;
+    const int M = (int)min((int64_t)128, p.M - m0);
+    const int N = p.N, K = p.K;
+    const int lr = tid >> 2, lc = (tid & 3) * 8;
+    bool aok[2], bok[2];
+    const float* pa[2];
+    const uint16_t* pw[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int rr = lr + 64 * h;
+        aok[h] = rr < M;
+        bok[h] = n0 + rr < N;
+        const int64_t arow = aok[h] ? (p.a_rows ? (int64_t)p.a_rows[m0 + rr] : m0 + rr) : 0;
+        pa[h] = p.A + b * p.a_batch + arow * p.lda;
+        pw[h] = (const uint16_t*)p.W + b * p.w_batch + (int64_t)(bok[h] ? n0 + rr : 0) * K;
+    }
+    const int64_t w2 = (int64_t)N * K;
+    float ra[2][8];
+    uint16_t rb[2][8], rb2[2][8];
+    auto gload = [&](int k0) {
+        const int k = k0 + lc;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (aok[h] && vecA && k + 8 <= K) {
+                const float4 u = *(const float4*)(pa[h] + k), v = *(const float4*)(pa[h] + k + 4);
+                ra[h][0] = u.x; ra[h][1] = u.y; ra[h][2] = u.z; ra[h][3] = u.w; ra[h][4] = v.x; ra[h][5] = v.y; ra[h][6] = v.z; ra[h][7] = v.w;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ra[h][i] = (aok[h] && k + i < K) ? pa[h][k + i] : 0.0f;
+            }
+            if (bok[h] && vecW && k + 8 <= K) {
+                *(uint4*)rb[h] = *(const uint4*)(pw[h] + k);
+                if (DUAL) *(uint4*)rb2[h] = *(const uint4*)(pw[h] + w2 + k);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    rb[h][i] = (bok[h] && k + i < K) ? pw[h][k + i] : (uint16_t)0;
+                    if (DUAL) rb2[h][i] = (bok[h] && k + i < K) ? pw[h][w2 + k + i] : (uint16_t)0;
+                }
+            }
+        }
+    };
+    auto lstore = [&](int buf) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            uint32_t w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[i] = dn_bf16_rne(ra[h][2 * i]) | (dn_bf16_rne(ra[h][2 * i + 1]) << 16);
+            *(uint4*)&sA[buf][lr + 64 * h][lc] = make_uint4(w[0], w[1], w[2], w[3]);
+            *(uint4*)&sB[buf][lr + 64 * h][lc] = *(const uint4*)rb[h];
+            if (DUAL) *(uint4*)&sB2[buf][lr + 64 * h][lc] = *(const uint4*)rb2[h];
+        }
+    };
+    dn_v4f acc[4][4], acc2[DUAL ? 4 : 1][DUAL ? 4 : 1];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[i][j] = dn_v4f{0, 0, 0, 0};
+            if (DUAL) acc2[DUAL ? i : 0][DUAL ? j : 0] = dn_v4f{0, 0, 0, 0};
+        }
+    const int fr = lane & 15, fk = lane >> 4;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    const int KT = (K + 31) / 32;
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < KT) gload((kt + 1) * 32);
+        dn_v8bf a[4], bb[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = *(const dn_v8bf*)&sA[cur][wm * 64 + i * 16 + fr][fk * 8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bb[j] = *(const dn_v8bf*)&sB[cur][wn * 64 + j * 16 + fr][fk * 8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], bb[j], acc[i][j], 0, 0, 0);
+        if (DUAL) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bb[j] = *(const dn_v8bf*)&sB2[cur][wn * 64 + j * 16 + fr][fk * 8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc2[DUAL ? i : 0][DUAL ? j : 0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], bb[j], acc2[DUAL ? i : 0][DUAL ? j : 0], 0, 0, 0);
+        }
+        if (kt + 1 < KT) lstore(cur ^ 1);
+        __syncthreads();
+    }
+    float* C = p.C + b * p.c_batch;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int reg = 0; reg < 4; ++reg) {
+            const int rl = wm * 64 + i * 16 + fk * 4 + reg;
+            if (rl >= M) continue;
+            const int64_t r = m0 + rl;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = n0 + wn * 64 + j * 16 + fr;
+                if (c < N) C[r * p.ldc + c] = dn_epilogue<EPI>(p, acc[i][j][reg], DUAL ? acc2[DUAL ? i : 0][DUAL ? j : 0][reg] : 0.0f, b, r, c);
             }
         }
 }
@@ -489,15 +611,19 @@ static void launch_tile(const i64h_linear& d, dim3 grid, hipStream_t s, int vecA
     }
 }
 
-static int g_skinny = 1, g_rows64 = 1;
+// the large tile is off by default: at 4096 rows and 1024 to 8192 columns (256 to 1024 tiles) it measured 1.3 to 1.8 times SLOWER than
+// the 64 x 64 kernel - one workgroup per CU leaves nothing to run while it waits at its barriers
+static int g_skinny = 1, g_rows64 = 1, g_tile128 = 0;
 
 extern "C" {
 
 // tuning / test knob, bit 0: launches of at most 8 rows on the weight-streaming kernel; bit 1: launches of at most 64 rows on the
-// fragment-streaming kernel (default 3: both; 0 = every launch on the tile kernel)
+// fragment-streaming kernel; bit 2: launches of 256 or more 128 x 128 tiles on the large-tile kernel (default 3; 0 = every launch on
+// the 64 x 64 tile kernel)
 int i64h_set_linear_skinny(int32_t on) {
     g_skinny = on & 1;
     g_rows64 = (on >> 1) & 1;
+    g_tile128 = (on >> 2) & 1;
     return 0;
 }
 
@@ -536,6 +662,18 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
             case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), 0, s, d); break;
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d); break;
             default: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_STORE>), grid, dim3(256), 0, s, d); break;
+        }
+        I64H_CHECK_LAUNCH();
+        return 0;
+    }
+    const int64_t tiles128 = ((d.N + 127) / 128) * ((d.M + 127) / 128) * (int64_t)d.batch;
+    if (g_tile128 && !d.exact && tiles128 >= 256) {     // at least a workgroup per CU: the large tile pays
+        const dim3 grid((unsigned)((d.N + 127) / 128), (unsigned)((d.M + 127) / 128), (unsigned)d.batch);
+        switch (d.epilogue) {
+            case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_GELU_MUL>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+            case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+            case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+            default: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_STORE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         }
         I64H_CHECK_LAUNCH();
         return 0;
