@@ -375,14 +375,14 @@ __global__ __launch_bounds__(256) void linear_skinny_kernel(const i64h_linear p,
 
 
 // ---------------------------------------------------------------------------------------------------------------------------
-// At most 64 rows (decode steps, small batches), bf16 form.  A workgroup owns 16 output columns; its four waves take every fourth
-// 32-wide k step, each with up to four 16-row blocks of A against the one weight fragment, all operands read straight from memory
+// At most 64 rows (decode steps, small batches), bf16 form.  A workgroup owns 16 output columns; its four or eight waves deal the
+// 32-wide k steps among them, each with up to four 16-row blocks of A against the one weight fragment, all operands read straight from memory
 // as matrix-core fragments (no staging, no barrier inside the loop); the four partial tiles meet in LDS, then the epilogue.
 // Many small workgroups fill the chip where a launch has few 64-column tiles, and the weights stream exactly once.
-template <int EPI>
-__global__ __launch_bounds__(256) void linear_rows64_kernel(const i64h_linear p) {
+template <int EPI, int NW>
+__global__ __launch_bounds__(64 * NW) void linear_rows64_kernel(const i64h_linear p) {
     constexpr bool DUAL = EPI == I64H_EPI_GELU_MUL;
-    __shared__ float red[DUAL ? 2 : 1][4][64][17];
+    __shared__ float red[DUAL ? 2 : 1][NW][64][17];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int n = lane & 15, kg = lane >> 4;
     const int64_t b = blockIdx.z;
@@ -408,27 +408,41 @@ __global__ __launch_bounds__(256) void linear_rows64_kernel(const i64h_linear p)
         acc2[i] = dn_v4f{0, 0, 0, 0};
     }
     const int KT = (K + 31) / 32;
-    for (int kt = wv; kt < KT; kt += 4) {
-        const int k = kt * 32 + kg * 8;
-        const bool kin = k < K;
-        uint4 wf = make_uint4(0, 0, 0, 0), wf2 = make_uint4(0, 0, 0, 0);
-        if (cok && kin) {
-            wf = *(const uint4*)(pw + k);
-            if (DUAL) wf2 = *(const uint4*)(pw2 + k);
-        }
+    // two k steps per turn: the loads of both are requested before the first matrix instruction
+    for (int kt = wv; kt < KT; kt += 2 * NW) {
+        uint4 wf[2], wf2[2], af[2][4];
+        float4 au[2][4], av[2][4];
+        bool kin[2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if (i < mblocks) {
-                uint4 af = make_uint4(0, 0, 0, 0);
-                if (rok[i] && kin) {
-                    const float4 u = *(const float4*)(pa[i] + k), v = *(const float4*)(pa[i] + k + 4);
-                    af = make_uint4(dn_bf16_rne(u.x) | (dn_bf16_rne(u.y) << 16), dn_bf16_rne(u.z) | (dn_bf16_rne(u.w) << 16),
-                                    dn_bf16_rne(v.x) | (dn_bf16_rne(v.y) << 16), dn_bf16_rne(v.z) | (dn_bf16_rne(v.w) << 16));
+        for (int h = 0; h < 2; ++h) {
+            const int k = (kt + h * NW) * 32 + kg * 8;
+            kin[h] = kt + h * NW < KT && k < K;
+            wf[h] = wf2[h] = make_uint4(0, 0, 0, 0);
+            if (cok && kin[h]) {
+                wf[h] = *(const uint4*)(pw + k);
+                if (DUAL) wf2[h] = *(const uint4*)(pw2 + k);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                au[h][i] = av[h][i] = make_float4(0, 0, 0, 0);
+                if (i < mblocks && rok[i] && kin[h]) {
+                    au[h][i] = *(const float4*)(pa[i] + k);
+                    av[h][i] = *(const float4*)(pa[i] + k + 4);
                 }
-                acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dn_v8bf, af), __builtin_bit_cast(dn_v8bf, wf), acc[i], 0, 0, 0);
-                if (DUAL) acc2[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dn_v8bf, af), __builtin_bit_cast(dn_v8bf, wf2), acc2[i], 0, 0, 0);
             }
         }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (i < mblocks) {
+                    const float4 u = au[h][i], v = av[h][i];
+                    af[h][i] = make_uint4(dn_bf16_rne(u.x) | (dn_bf16_rne(u.y) << 16), dn_bf16_rne(u.z) | (dn_bf16_rne(u.w) << 16),
+                                          dn_bf16_rne(v.x) | (dn_bf16_rne(v.y) << 16), dn_bf16_rne(v.z) | (dn_bf16_rne(v.w) << 16));
+                    acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dn_v8bf, af[h][i]), __builtin_bit_cast(dn_v8bf, wf[h]), acc[i], 0, 0, 0);
+                    if (DUAL) acc2[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(dn_v8bf, af[h][i]), __builtin_bit_cast(dn_v8bf, wf2[h]), acc2[i], 0, 0, 0);
+                }
+            }
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -439,12 +453,15 @@ __global__ __launch_bounds__(256) void linear_rows64_kernel(const i64h_linear p)
         }
     __syncthreads();
     float* C = p.C + b * p.c_batch;
-    for (int e = tid; e < 64 * 16; e += 256) {
+    for (int e = tid; e < 64 * 16; e += 64 * NW) {
         const int m = e >> 4, c = e & 15;
         if (m >= M || n0 + c >= N) continue;
-        const float s = ((red[0][0][m][c] + red[0][1][m][c]) + red[0][2][m][c]) + red[0][3][m][c];
-        float s2 = 0.0f;
-        if (DUAL) s2 = ((red[DUAL ? 1 : 0][0][m][c] + red[DUAL ? 1 : 0][1][m][c]) + red[DUAL ? 1 : 0][2][m][c]) + red[DUAL ? 1 : 0][3][m][c];
+        float s = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            s += red[0][w][m][c];
+            if (DUAL) s2 += red[DUAL ? 1 : 0][w][m][c];
+        }
         C[(int64_t)m * p.ldc + n0 + c] = dn_epilogue<EPI>(p, s, s2, b, m, n0 + c);
     }
 }
@@ -658,10 +675,11 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
     if (g_rows64 && !d.exact && d.M <= 64 && vecA && vecW) {
         const dim3 grid((unsigned)((d.N + 15) / 16), 1, (unsigned)d.batch);
         switch (d.epilogue) {
-            case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_GELU_MUL>), grid, dim3(256), 0, s, d); break;
-            case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), 0, s, d); break;
-            case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d); break;
-            default: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_STORE>), grid, dim3(256), 0, s, d); break;
+            // eight waves share the k steps where one accumulator is kept (the gate / up pair needs twice the LDS: four)
+            case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_GELU_MUL, 4>), grid, dim3(256), 0, s, d); break;
+            case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_MUL_SIGMOID, 8>), grid, dim3(512), 0, s, d); break;
+            case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SOFTCAP, 8>), grid, dim3(512), 0, s, d); break;
+            default: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_STORE, 8>), grid, dim3(512), 0, s, d); break;
         }
         I64H_CHECK_LAUNCH();
         return 0;
