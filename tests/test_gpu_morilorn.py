@@ -142,9 +142,9 @@ def test_gated_postnorm_and_depth_mix(dev, W, groups):
     mw = torch.randn(idx + 1, generator=g)
     hd = hist.to(dev)
     out, mix = torch.empty(n, W, device=dev), torch.empty(n, W, device=dev)
-    D.gated_postnorm(x.to(dev), nw.to(dev), groups, 1e-3, alpha=2.5, y=y.to(dev), ldy=W + 2, gate_pre=gp.to(dev), gate_off=4, ldg=W + 7, gate_bias=b.to(dev),
+    D.gated_postnorm(x.to(dev), nw.to(dev), groups, 1e-3, alpha=1.75, y=y.to(dev), ldy=W + 2, gate_pre=gp.to(dev), gate_off=4, ldg=W + 7, gate_bias=b.to(dev),
                      out=out, hist=hd, hist_index=idx, mix_w=mw.to(dev), mix_out=mix)
-    v = 2.5 * x.double() + torch.sigmoid(gp[:, 4:4 + W].double() + b.double()) * y[:, :W].double()
+    v = 1.75 * x.double() + torch.sigmoid(gp[:, 4:4 + W].double() + b.double()) * y[:, :W].double()
     ref = R.rms_norm(v, nw.double(), 1e-3, groups)
     assert torch.allclose(out.cpu().double(), ref, atol=2e-6, rtol=2e-6)
     assert torch.allclose(hd[idx].cpu().double(), ref, atol=2e-6, rtol=2e-6) and torch.equal(hd[idx + 1].cpu(), hist[idx + 1])
@@ -213,7 +213,7 @@ def test_latent_prep_norm_rotation_and_cache_write(dev, cache_dtype, H, d, e, r,
     from vllm_i64_amd import ops_dense as D
     from vllm_i64_amd.morilorn import inverse_frequencies
     g = torch.Generator().manual_seed(5)
-    T, base, eps = 37, 50000.0, 1e-4
+    T, base, eps = 37, 30000.0, 1e-4
     q_off, dkv_off = 3, 3 + H * (d + e) + 2
     P = torch.randn(T, dkv_off + r + e + 1, generator=g)
     nw = torch.randn(r, generator=g)
@@ -247,7 +247,7 @@ def _ref_attn(Q, rows, positions, window, scale, r):
 
 
 @pytest.mark.parametrize("cache_dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("window", [0, 1, 7, 16, 17, 40])
+@pytest.mark.parametrize("window", [0, 1, 7, 16, 17, 45])
 @pytest.mark.parametrize("r,e", [(32, 8), (20, 6)])   # widths the matrix-core form takes (multiples of 16 and 8), and widths it leaves to the row form
 def test_latent_attn_one_key_stands_out(dev, cache_dtype, window, r, e):
     """One cached row is made to dominate every head's softmax wherever it is visible.  It is placed far back, at page borders and
