@@ -506,6 +506,42 @@ __global__ __launch_bounds__(256) void gated_postnorm_kernel(const i64h_postnorm
     }
     __syncthreads();
     const int64_t plane = p.n * (int64_t)W;
+    if ((W & 3) == 0 && ((uintptr_t)p.norm_w & 15) == 0 && ((uintptr_t)p.out & 15) == 0 && ((uintptr_t)p.hist & 15) == 0 && ((uintptr_t)p.mix_out & 15) == 0 &&
+        gs % 4 == 0) {
+        // four columns per thread and 16-byte accesses; the history planes are read four at a time (independent loads in flight)
+        for (int c = tid * 4; c < W; c += 1024) {
+            const float den = sv[W + c / gs];
+            const float4 nw = *(const float4*)(p.norm_w + c);
+            float4 o;
+            o.x = sv[c] / den * nw.x; o.y = sv[c + 1] / den * nw.y; o.z = sv[c + 2] / den * nw.z; o.w = sv[c + 3] / den * nw.w;
+            if (p.out) *(float4*)(p.out + m * W + c) = o;
+            if (p.mix_w) {
+                const float* h = p.hist + m * W + c;
+                *(float4*)(p.hist + p.hist_index * plane + m * W + c) = o;
+                float4 a = make_float4(0, 0, 0, 0);
+                int j = 0;
+                for (; j + 4 <= p.hist_index; j += 4) {
+                    float4 v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) v[u] = *(const float4*)(h + (j + u) * plane);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const float wj = p.mix_w[j + u];
+                        a.x += wj * v[u].x; a.y += wj * v[u].y; a.z += wj * v[u].z; a.w += wj * v[u].w;
+                    }
+                }
+                for (; j < p.hist_index; ++j) {
+                    const float4 v = *(const float4*)(h + j * plane);
+                    const float wj = p.mix_w[j];
+                    a.x += wj * v.x; a.y += wj * v.y; a.z += wj * v.z; a.w += wj * v.w;
+                }
+                const float wl = p.mix_w[p.hist_index];
+                a.x += wl * o.x; a.y += wl * o.y; a.z += wl * o.z; a.w += wl * o.w;
+                *(float4*)(p.mix_out + m * W + c) = a;
+            }
+        }
+        return;
+    }
     for (int c = tid; c < W; c += 256) {
         const float o = sv[c] / sv[W + c / gs] * p.norm_w[c];
         if (p.out) p.out[m * W + c] = o;
