@@ -140,6 +140,7 @@ typedef struct {
     int32_t splits;      /* mode 2: every token's keys are dealt to this many waves (tiles of 32 keys in turn) and merged by a second launch */
     float* workspace;    /* i64h_latent_attn_workspace_floats(n, heads, kv_rank, splits) floats when splits > 1 (NULL: no split) */
 } i64h_latent_attn_args;
+int i64h_set_latent_attn_decode_form(int32_t on); /* tuning / test knob: 1 (default) = mode 2 launches run the kernel that requests a tile's fragments a tile ahead; 0 = the general matrix-core kernel; same results up to summation order */
 int64_t i64h_latent_attn_workspace_floats(int64_t n, int32_t heads, int32_t kv_rank, int32_t splits);
 int i64h_latent_attn(const i64h_latent_attn_args* d, void* stream);
 

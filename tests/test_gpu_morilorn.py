@@ -310,11 +310,14 @@ def test_latent_attn_keys_dealt_to_several_waves(dev):
     pos = torch.tensor([t - 1 for t in lens], dtype=torch.int32)
     for window in (0, 100):
         ref = torch.cat([_ref_attn(Q[i:i + 1], rows_of[i], [lens[i] - 1], window, 0.4, r) for i in range(4)])
-        for splits in (1, 2, 5, 64):
-            out = torch.empty(4, H, r, device=dev)
-            D.latent_attn(Q.to(dev), cache, bt.to(dev), torch.arange(4, dtype=torch.int32, device=dev), pos.to(dev), window=window, scale=0.4, heads=H,
-                          kv_rank=r, rot_dim=e, out=out, mode=2, splits=splits)
-            assert torch.allclose(out.cpu().double(), ref, atol=1e-3, rtol=1e-3), (window, splits)
+        for form in (1, 0):      # the kernel that requests its fragments a tile ahead, and the general matrix-core kernel
+            D.call_dense("i64h_set_latent_attn_decode_form", form)
+            for splits in (1, 2, 5, 64):
+                out = torch.empty(4, H, r, device=dev)
+                D.latent_attn(Q.to(dev), cache, bt.to(dev), torch.arange(4, dtype=torch.int32, device=dev), pos.to(dev), window=window, scale=0.4, heads=H,
+                              kv_rank=r, rot_dim=e, out=out, mode=2, splits=splits)
+                assert torch.allclose(out.cpu().double(), ref, atol=1e-3, rtol=1e-3), (window, splits, form)
+    D.call_dense("i64h_set_latent_attn_decode_form", 1)
 
 
 def test_sample_rows(dev):

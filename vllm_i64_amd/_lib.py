@@ -209,6 +209,7 @@ DENSE_LIB_PATH = os.path.join(_HERE, "libi64hip_dense.so")
 DENSE_SIGNATURES: Dict[str, str] = {
     "i64h_linear_run": "pp",
     "i64h_set_linear_skinny": "i",
+    "i64h_set_latent_attn_decode_form": "i",
     "i64h_embed_scaled": "ppfplilp",
     "i64h_gated_postnorm": "pp",
     "i64h_latent_prep": "pp",

@@ -19,10 +19,8 @@
 typedef float dn_v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 dn_v8bf __attribute__((ext_vector_type(8)));
 
-__device__ __forceinline__ uint32_t dn_bf16_rne(float f) {  // round to nearest even; NaN stays NaN
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+__device__ __forceinline__ uint32_t dn_bf16_rne(float f) {  // round to nearest even, NaN stays NaN: the hardware conversion of this chip
+    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ float dn_bf16_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 __device__ __forceinline__ float dn_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }

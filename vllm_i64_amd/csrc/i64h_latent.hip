@@ -163,9 +163,8 @@ __global__ __launch_bounds__(256) void latent_attn_row_kernel(const i64h_latent_
 typedef __bf16 lt_v8bf __attribute__((ext_vector_type(8)));
 typedef float lt_v4f __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ uint32_t lt_rne(float f) {
-    const uint32_t u = __float_as_uint(f);
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+__device__ __forceinline__ uint32_t lt_rne(float f) {  // nearest even: the hardware conversion of this chip
+    return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ void lt_split(float x, uint32_t& hi, uint32_t& lo) {
     hi = lt_rne(x);
@@ -349,6 +348,177 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     }
 }
 
+// The same products for rows that are one per sequence (every wave: one token, 16 heads, a share of the keys), arranged around the
+// memory latency that dominates such launches: a tile's 18 fragment loads are requested together, the NEXT tile's are requested as
+// soon as this tile's scores and transposed columns are done - under its softmax and second product - and the cache rows of the tile
+// after that are looked up a tile ahead.  The workgroup is one wave, so LDS traffic needs program order only (no barrier, whose
+// fence would wait for the loads in flight).  Registers: a whole SIMD's (one wave per SIMD is all such a launch has anyway).
+__global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_latent_attn_args p, const int splits) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int lane = threadIdx.x, n = lane & 15, kg = lane >> 4;
+    const int r = p.kv_rank, D = r + p.rot_dim, H = p.heads, bs = p.block_size, win = p.window;
+    uint16_t* Vt = (uint16_t*)smem;
+    uint16_t* Ph = Vt + r * LT_VLD;
+    uint16_t* Pl = Ph + 16 * LT_VLD;
+    int* rowoff = (int*)(Pl + 16 * LT_VLD);   // [2][32] cache rows of two tiles' keys
+    const int64_t task = blockIdx.x;
+    const int split = blockIdx.y;
+    const int hgroups = (H + 15) / 16;
+    const int64_t tok = task / hgroups;
+    const int head0 = (int)(task % hgroups) * 16;
+    const int pos = p.positions[tok], slot = p.slot_ids[tok];
+    const int lo = win > 0 ? max(0, pos - win + 1) : 0, hi = pos;
+    const int32_t* bt = p.block_table + (int64_t)slot * p.max_blocks_per_seq;
+    const uint16_t* cache = (const uint16_t*)p.cache;
+    const int step = 32 * splits;
+    const int kb0 = (lo & ~31) + 32 * split;
+    auto lookup = [&](int kb, int buf) {
+        if (lane < 32) {
+            const int jc = min(kb + lane, hi);
+            rowoff[buf * 32 + lane] = bt[jc / bs] * bs + jc % bs;
+        }
+    };
+    uint4 kf[2][LT_KD];
+    auto request = [&](int buf) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const uint16_t* rowp = cache + (int64_t)rowoff[buf * 32 + 16 * b + n] * D;
+#pragma unroll
+            for (int ks = 0; ks < LT_KD; ++ks) {
+                const int d0 = ks * 32 + kg * 8;
+                kf[b][ks] = (ks * 32 < D && d0 < D) ? *(const uint4*)(rowp + d0) : make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+    if (kb0 <= hi) {
+        lookup(kb0, 0);
+        if (kb0 + step <= hi) lookup(kb0 + step, 1);
+        __builtin_amdgcn_wave_barrier();
+        request(0);
+    }
+    // the query of row n (head head0 + n) times scale * log2(e), as two bf16 terms - converted while the first tile travels
+    uint4 Qh[LT_KD], Ql[LT_KD];
+    {
+        const bool valid_n = head0 + n < H;
+        const float* q = p.Q + (tok * H + head0 + n) * D;
+        const float qs = p.scale * 1.4426950408889634f;
+#pragma unroll
+        for (int ks = 0; ks < LT_KD; ++ks) {
+            const int d0 = ks * 32 + kg * 8;
+            uint32_t h[8], l[8];
+            if (valid_n && d0 < D) {
+                const float4 a = *(const float4*)(q + d0), b = *(const float4*)(q + d0 + 4);
+                const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) lt_split(v[i] * qs, h[i], l[i]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) h[i] = l[i] = 0;
+            }
+            Qh[ks] = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+            Ql[ks] = make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16));
+        }
+    }
+    lt_v4f acc[LT_NB];
+#pragma unroll
+    for (int nb = 0; nb < LT_NB; ++nb) acc[nb] = lt_v4f{0, 0, 0, 0};
+    float mrow[4], lrow[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        mrow[g] = -INFINITY;
+        lrow[g] = 0.0f;
+    }
+    int it = 0;
+    for (int kb = kb0; kb <= hi; kb += step, ++it) {
+        const int cur = it & 1;
+        lt_v4f S[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            S[b] = lt_v4f{0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < LT_KD; ++ks) {
+                if (ks * 32 < D) {
+                    const int d0 = ks * 32 + kg * 8;
+                    const uint4 f = kf[b][ks];
+                    S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Qh[ks]), __builtin_bit_cast(lt_v8bf, f), S[b], 0, 0, 0);
+                    S[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, Ql[ks]), __builtin_bit_cast(lt_v8bf, f), S[b], 0, 0, 0);
+                    if (d0 < r) {
+                        const uint32_t kw[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+                        for (int c = 0; c < 8; ++c) Vt[(d0 + c) * LT_VLD + 16 * b + n] = (uint16_t)(kw[c >> 1] >> (16 * (c & 1)));
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (kb + step <= hi) request(cur ^ 1);          // the next tile travels under this tile's softmax and second product
+        float al[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int rr = kg * 4 + g;
+            float sv[2];
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int j = kb + 16 * b + n;
+                sv[b] = (j <= pos && j >= lo) ? S[b][g] : -INFINITY;
+            }
+            const float mx = row16_max(fmaxf(sv[0], sv[1]));
+            const float mn = fmaxf(mrow[g], mx);
+            const float ms = mn == -INFINITY ? 0.0f : mn;
+            al[g] = __builtin_amdgcn_exp2f(mrow[g] - ms);
+            const float p0 = __builtin_amdgcn_exp2f(sv[0] - ms), p1 = __builtin_amdgcn_exp2f(sv[1] - ms);
+            lrow[g] = lrow[g] * al[g] + group_sum(p0 + p1, 16);
+            mrow[g] = mn;
+            uint32_t h0, l0, h1, l1;
+            lt_split(p0, h0, l0);
+            lt_split(p1, h1, l1);
+            Ph[rr * LT_VLD + n] = (uint16_t)h0;
+            Pl[rr * LT_VLD + n] = (uint16_t)l0;
+            Ph[rr * LT_VLD + 16 + n] = (uint16_t)h1;
+            Pl[rr * LT_VLD + 16 + n] = (uint16_t)l1;
+        }
+        __builtin_amdgcn_wave_barrier();
+        const uint4 pah = *(const uint4*)&Ph[n * LT_VLD + kg * 8], pal = *(const uint4*)&Pl[n * LT_VLD + kg * 8];
+#pragma unroll
+        for (int nb = 0; nb < LT_NB; ++nb) {
+            if (nb * 16 < r) {
+                const uint4 vf = *(const uint4*)&Vt[(nb * 16 + n) * LT_VLD + kg * 8];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) acc[nb][g] *= al[g];
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, pah), __builtin_bit_cast(lt_v8bf, vf), acc[nb], 0, 0, 0);
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(lt_v8bf, pal), __builtin_bit_cast(lt_v8bf, vf), acc[nb], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (kb + 2 * step <= hi) lookup(kb + 2 * step, cur);   // rows of the tile after next, into the buffer this tile is done with
+    }
+    if (splits > 1) {
+        float* w = p.workspace + ((int64_t)task * splits + split) * 16 * (r + 2);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            float* o = w + (kg * 4 + g) * (r + 2);
+#pragma unroll
+            for (int nb = 0; nb < LT_NB; ++nb)
+                if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g];
+            if (n == 0) {
+                o[r] = mrow[g];
+                o[r + 1] = lrow[g];
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const int head = head0 + kg * 4 + g;
+        if (head >= H) continue;
+        float* o = p.out + (tok * H + head) * r;
+        const float inv = 1.0f / lrow[g];
+#pragma unroll
+        for (int nb = 0; nb < LT_NB; ++nb)
+            if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g] * inv;
+    }
+}
+
 // the shares of a token's keys, merged: one wave per (token, head); lane s holds share s's maximum and weight sum (at most 64
 // shares), then every lane sums its columns over the shares, eight loads in flight at a time
 __global__ __launch_bounds__(64) void latent_attn_merge_kernel(const i64h_latent_attn_args p, const int splits) {
@@ -397,6 +567,12 @@ int i64h_latent_prep(const i64h_latent_prep_args* dp, void* stream) {
     return 0;
 }
 
+static int g_decode_form = 1;
+int i64h_set_latent_attn_decode_form(int32_t on) {  // tuning / test knob: 0 = rows that are one per sequence on the general matrix-core kernel
+    g_decode_form = on;
+    return 0;
+}
+
 int64_t i64h_latent_attn_workspace_floats(int64_t n, int32_t heads, int32_t kv_rank, int32_t splits) {
     if (splits <= 1) return 0;
     return n * ((heads + 15) / 16) * (int64_t)(splits > 64 ? 64 : splits) * 16 * (kv_rank + 2);
@@ -419,7 +595,10 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
         I64H_CHECK_ARG(tasks < (1ll << 31), "latent_attn: too many tiles");
         const int splits = (!row_tiles && d.workspace && d.splits > 1) ? (d.splits > 64 ? 64 : d.splits) : 1;
         const size_t bytes = (size_t)d.kv_rank * LT_VLD * 2 + 2 * 16 * LT_VLD * 2 + 64 * 4;
-        hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, row_tiles, splits);
+        if (row_tiles || !g_decode_form)
+            hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, row_tiles, splits);
+        else
+            hipLaunchKernelGGL(latent_attn_mfma_decode_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, splits);
         I64H_CHECK_LAUNCH();
         if (splits > 1) {
             hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tasks, 16), dim3(64), 0, (hipStream_t)stream, d, splits);
