@@ -287,10 +287,11 @@ def test_latent_attn_one_key_stands_out(dev, cache_dtype, window, r, e):
                 assert close == sees, (window, star, p)
 
 
-def test_latent_attn_keys_dealt_to_several_waves(dev):
-    """Decode rows whose keys are split over waves and merged: same result as one wave per token, also when some shares are empty."""
+@pytest.mark.parametrize("H,r,e", [(5, 48, 16), (16, 256, 32), (18, 240, 80)])    # the last two: the widest rows the matrix-core forms take
+def test_latent_attn_keys_dealt_to_several_waves(dev, H, r, e):
+    """Decode rows whose keys are split over waves and merged: same result as one wave per token, also when some shares are empty;
+    and the same rows through the form made for prompt portions."""
     from vllm_i64_amd import ops_dense as D
-    H, r, e = 5, 48, 16
     g = torch.Generator().manual_seed(2)
     lens = [1, 40, 333, 64]
     nb = [(t + 15) // 16 for t in lens]
@@ -317,6 +318,10 @@ def test_latent_attn_keys_dealt_to_several_waves(dev):
                 D.latent_attn(Q.to(dev), cache, bt.to(dev), torch.arange(4, dtype=torch.int32, device=dev), pos.to(dev), window=window, scale=0.4, heads=H,
                               kv_rank=r, rot_dim=e, out=out, mode=2, splits=splits)
                 assert torch.allclose(out.cpu().double(), ref, atol=1e-3, rtol=1e-3), (window, splits, form)
+        out = torch.empty(4, H, r, device=dev)
+        D.latent_attn(Q.to(dev), cache, bt.to(dev), torch.arange(4, dtype=torch.int32, device=dev), pos.to(dev), window=window, scale=0.4, heads=H,
+                      kv_rank=r, rot_dim=e, out=out, mode=3)
+        assert torch.allclose(out.cpu().double(), ref, atol=1e-3, rtol=1e-3), (window, "row tiles")
     D.call_dense("i64h_set_latent_attn_decode_form", 1)
 
 
