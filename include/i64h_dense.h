@@ -27,13 +27,16 @@ int i64h_device_check(void);
  * exact = 1: W is widened to fp32 while it is staged, products on v_mfma_f32_16x16x4_f32: true 32-bit arithmetic.
  * epilogue: I64H_EPI_STORE; I64H_EPI_GELU_MUL: gelu_tanh(A W^T) * (A W2^T) with W2 = W + N * K (gate rows, then up rows);
  *   I64H_EPI_MUL_SIGMOID: * sigmoid(E[b][m, n]) (E fp32, row stride lde, batch stride e_batch);
- *   I64H_EPI_SOFTCAP: cap * tanh(. / cap).
+ *   I64H_EPI_SOFTCAP: cap * tanh(. / cap);  I64H_EPI_GELU_ERF: 0.5 v (1 + erf(v / sqrt 2));  I64H_EPI_SCALE: v * scale.
+ *   bias (may be NULL; fp32 [N], batch stride bias_batch) is added to the sum before any epilogue but I64H_EPI_GELU_MUL.
  * Any M, N, K >= 1; 16-byte loads are used where strides and addresses allow, element loads otherwise.
  * Launches with M <= I64H_SKINNY_ROWS take a weight-streaming form (one wave per output column group). */
 #define I64H_EPI_STORE 0
 #define I64H_EPI_GELU_MUL 1
 #define I64H_EPI_MUL_SIGMOID 2
 #define I64H_EPI_SOFTCAP 3
+#define I64H_EPI_GELU_ERF 4
+#define I64H_EPI_SCALE 5
 #define I64H_SKINNY_ROWS 8
 typedef struct {
     const float* A;
@@ -51,6 +54,9 @@ typedef struct {
     const float* E;
     int64_t lde, e_batch;
     float softcap;
+    const float* bias;
+    int64_t bias_batch;
+    float scale;
 } i64h_linear;
 int i64h_linear_run(const i64h_linear* d, void* stream);
 
@@ -143,6 +149,194 @@ typedef struct {
 int i64h_set_latent_attn_decode_form(int32_t on); /* tuning / test knob: 1 (default) = mode 2 launches run the kernel that requests a tile's fragments a tile ahead; 0 = the general matrix-core kernel; same results up to summation order */
 int64_t i64h_latent_attn_workspace_floats(int64_t n, int32_t heads, int32_t kv_rank, int32_t splits);
 int i64h_latent_attn(const i64h_latent_attn_args* d, void* stream);
+
+/* ==== recurrent and hybrid layers ==========================================================================================
+ * Rows of a step are in sequence order: the rows of one sequence are consecutive and carry consecutive positions.  Row t
+ * continues row t - 1 iff slot_ids[t - 1] == slot_ids[t] and positions[t - 1] + 1 == positions[t].  A sequence's state lives in
+ * its slot; a row at position 0 starts from the empty state whatever the slot held before (a slot that is used again needs no
+ * clearing).  seg_start [nseg + 1] lists the first row of every run of consecutive rows of one sequence (seg_start[nseg] = n). */
+
+/* ---- token embedding + hashed bigram embedding ----------------------------------------------------------------------------------
+ * out[c][t, :] = table[ids[t]] + bigram[row(t)] for c < copies (out fp32 [copies, n, W]);  row(t) = buckets at position 0, else
+ * (previous * mul_prev + ids[t] * mul_cur) mod buckets, previous = the token of the row before in the same sequence, or
+ * prev_token[slot] (the last token of the sequence's earlier steps).  A second launch stores every sequence's last token of
+ * this step in prev_token.  bigram == NULL: the token embedding alone.  Tables bf16. */
+typedef struct {
+    const int64_t* ids;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    const void* table;
+    int64_t V;
+    int32_t W;
+    const void* bigram;
+    int64_t buckets, mul_prev, mul_cur;
+    int64_t* prev_token;
+    float* out;
+    int32_t copies;
+    int64_t n;
+} i64h_embed_bigram_args;
+int i64h_embed_bigram(const i64h_embed_bigram_args* d, void* stream);
+
+/* ---- multi-stream residual (hyper-connections) with the next sublayer's RMS norm -------------------------------------------------
+ * streams fp32 [S, n, W], updated in place, one workgroup per row:
+ *   write (y != NULL):  v = y2 ? 0.5 * (rms(y) * yn_w + rms(y2) * y2n_w) : y      (rms over the W columns with y_eps; weights [W])
+ *                       new_t = sum_s mix[s * S + t] * old_s + out_w[t] * v          (mix == NULL: new_t = old_t + out_w[t] * v)
+ *   read  (h != NULL):  u = sum_s in_w[s] * x_s  (in_w == NULL: the plain sum);  h = u / sqrt(mean(u^2) + eps) * norm_w[c % norm_w_len]
+ * rows (may be NULL, read only launches): h[m] is computed from row rows[m] of the streams (the rows whose logits are wanted). */
+typedef struct {
+    float* streams;
+    int32_t S;
+    int64_t n;
+    int32_t W;
+    const float* y;
+    int64_t ldy;
+    const float* y2;
+    int64_t ldy2;
+    const float* yn_w;
+    const float* y2n_w;
+    float y_eps;
+    const float* mix;
+    const float* out_w;
+    const float* in_w;
+    const float* norm_w;
+    int32_t norm_w_len;
+    float eps;
+    float* h;
+    const int32_t* rows;
+    int64_t m_rows;
+} i64h_streams_args;
+int i64h_streams_step(const i64h_streams_args* d, void* stream);
+
+/* ---- causal per-channel convolution with carried inputs + silu ---------------------------------------------------------------------
+ * out[t, c] = silu(bias[c] + sum_k w[c, k] * in(t, taps - 1 - k)),  in(t, d) = the input of channel c d positions before row t:
+ * zero before position 0, a row of this step where the sequence has one there, else the carried inputs state fp32
+ * [slots, taps - 1, channels] (the last taps - 1 inputs of the sequence's earlier steps, oldest first).  Inputs are the columns
+ * [off, off + channels) of P.  A second launch stores the new carried inputs.  w fp32 [channels, taps]. */
+typedef struct {
+    const float* P;
+    int64_t ldp;
+    int32_t off, channels, taps;
+    const float* w;
+    const float* bias;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    float* state;
+    float* out;
+    int64_t ldo;
+    int64_t n;
+} i64h_causal_conv_args;
+int i64h_causal_conv(const i64h_causal_conv_args* d, void* stream);
+
+/* ---- selective state-space recurrence (scalar decay per head) ---------------------------------------------------------------------
+ * Per sequence and head a (state x vdim) matrix S in fp32:  dt = softplus(dt_raw + dt_bias[a]),
+ *   S <- exp(-exp(A_log[a]) * dt) * S + dt * B_t x_t^T,   y_t = S^T C_t + Dskip[a] * x_t,
+ * x_t = xbc[t, a * vdim : +vdim], B_t = xbc[t, heads * vdim + g * state : +state], C_t = xbc[t, heads * vdim + (groups + g) * state : +state],
+ * g = a / (heads / groups), dt_raw = dt[t, a].  ssm_state fp32 [slots, heads, state, vdim].  All arithmetic fp32. */
+typedef struct {
+    const float* xbc;
+    int64_t ldx;
+    const float* dt;
+    int64_t lddt;
+    const float* dt_bias;
+    const float* A_log;
+    const float* Dskip;
+    int32_t heads, vdim, state, groups;
+    const int32_t* seg_start;
+    int32_t nseg;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    float* ssm_state;
+    float* y;
+    int64_t ldy;
+    int64_t n;
+} i64h_ssm_scan_args;
+int i64h_ssm_scan(const i64h_ssm_scan_args* d, void* stream);
+
+/* out[t, :] = rms_groups(y[t, :] * silu(z[t, :])) * w: the `width` columns in `groups` equal consecutive parts, each divided by
+ * sqrt(mean(part^2) + eps).  z == NULL: no gate. */
+typedef struct {
+    const float* y;
+    int64_t ldy;
+    const float* z;
+    int64_t ldz;
+    const float* w;
+    int32_t width, groups;
+    float eps;
+    float* out;
+    int64_t ldo;
+    int64_t n;
+} i64h_gate_norm_args;
+int i64h_gate_norm(const i64h_gate_norm_args* d, void* stream);
+
+/* ---- minimal gated recurrence ------------------------------------------------------------------------------------------------------
+ * Per sequence and channel c < width, fp32:  z = sigmoid(P[t, z_off + c]),  u = P[t, x_off + c],
+ *   cand = u >= 0 ? u + 0.5 : sigmoid(u),   S <- (1 - z) * S + z * cand,   out[t, c] = S * silu(P[t, g_off + c]).
+ * state fp32 [slots, width]. */
+typedef struct {
+    const float* P;
+    int64_t ldp;
+    int32_t z_off, x_off, g_off, width;
+    const int32_t* seg_start;
+    int32_t nseg;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    float* state;
+    float* out;
+    int64_t ldo;
+    int64_t n;
+} i64h_mingru_scan_args;
+int i64h_mingru_scan(const i64h_mingru_scan_args* d, void* stream);
+
+/* ---- attention whose values are the keys ---------------------------------------------------------------------------------------------
+ * One cached row per token and layer: the kv_heads * dim key values as projected (fp32, cache_dtype 0, or bf16, 2), plus one fp32
+ * number per token, kscale = 1 / sqrt(mean(row^2) + eps); paged as the latent cache above.
+ * i64h_kattn_prep, per row t of the projections P:  q = P[t, q_off : + heads * dim], k = P[t, k_off : + kv_heads * dim];
+ *   Q[t, h, d] = q[h, d] / sqrt(mean(q^2) + eps) * q_norm_w[h * dim + d] * k_norm_w[g * dim + d] * scale * temp[h]
+ *   (means over the whole row; g = h / (heads / kv_heads); temp may be NULL), cache row <- k, kscale <- 1 / sqrt(mean(k^2) + eps).
+ * With these a score against the normed key is Q[t, h] . k_j * kscale_j. */
+typedef struct {
+    const float* P;
+    int64_t ldp;
+    int32_t q_off, k_off;
+    int32_t heads, kv_heads, dim;
+    const float* q_norm_w;
+    const float* k_norm_w;
+    const float* temp;
+    float scale, eps;
+    const int32_t* positions;
+    const int32_t* slot_ids;
+    const int32_t* block_table;
+    int32_t max_blocks_per_seq, block_size;
+    void* cache;
+    int32_t cache_dtype;
+    float* kscale;
+    float* Q;
+    int64_t n;
+} i64h_kattn_prep_args;
+int i64h_kattn_prep(const i64h_kattn_prep_args* d, void* stream);
+
+/* i64h_kattn: row t (position p) sees the cached positions j <= p of its sequence with j / chunk == p / chunk (chunk <= 0: all);
+ *   s_j = Q[t, h] . k_j * kscale_j + bias[min(p - j, bias_rows - 1) * heads + h]      (bias fp32 [bias_rows, heads], may be NULL)
+ *   w_j = exp(s_j) / (sink + sum_i exp(s_i))    (sink = 1: one more score of zero that carries no value; 0: the ordinary softmax)
+ *   out[t, h, :] = sum_j w_j * k_j[g, :].   Scores, weights and sums fp32.  out fp32 [n, heads, dim]. */
+typedef struct {
+    const float* Q;
+    const void* cache;
+    int32_t cache_dtype;
+    const float* kscale;
+    const int32_t* block_table;
+    int32_t max_blocks_per_seq, block_size;
+    const int32_t* slot_ids;
+    const int32_t* positions;
+    int32_t chunk;
+    const float* bias;
+    int32_t bias_rows;
+    int32_t sink;
+    float* out;
+    int64_t n;
+    int32_t heads, kv_heads, dim;
+} i64h_kattn_args;
+int i64h_kattn(const i64h_kattn_args* d, void* stream);
 
 /* ---- sampling --------------------------------------------------------------------------------------------------------------
  * out[r] = a token drawn from row r of logits fp32 [rows, V]: temperature[r] <= 0 -> the first index of the maximum (greedy);

@@ -215,6 +215,14 @@ DENSE_SIGNATURES: Dict[str, str] = {
     "i64h_latent_prep": "pp",
     "i64h_latent_attn": "pp",
     "i64h_sample_rows": "pplippppp",
+    "i64h_embed_bigram": "pp",
+    "i64h_streams_step": "pp",
+    "i64h_causal_conv": "pp",
+    "i64h_ssm_scan": "pp",
+    "i64h_gate_norm": "pp",
+    "i64h_mingru_scan": "pp",
+    "i64h_kattn_prep": "pp",
+    "i64h_kattn": "pp",
 }
 
 
@@ -222,7 +230,7 @@ class Linear(ctypes.Structure):
     """Mirror of i64h_linear (include/i64h_dense.h)."""
     _fields_ = [("A", _P), ("lda", _L), ("a_rows", _P), ("W", _P), ("C", _P), ("ldc", _L), ("M", _L), ("N", _I), ("K", _I), ("batch", _I),
                 ("a_batch", _L), ("w_batch", _L), ("c_batch", _L), ("exact", _I), ("epilogue", _I), ("E", _P), ("lde", _L), ("e_batch", _L),
-                ("softcap", _F)]
+                ("softcap", _F), ("bias", _P), ("bias_batch", _L), ("scale", _F)]
 
 
 class PostNorm(ctypes.Structure):
@@ -244,6 +252,57 @@ class LatentAttn(ctypes.Structure):
     _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("slot_ids", _P), ("positions", _P), ("window", _I), ("scale", _F), ("out", _P), ("n", _L), ("heads", _I), ("kv_rank", _I),
                 ("rot_dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P)]
+
+
+class EmbedBigram(ctypes.Structure):
+    """Mirror of i64h_embed_bigram_args (include/i64h_dense.h)."""
+    _fields_ = [("ids", _P), ("positions", _P), ("slot_ids", _P), ("table", _P), ("V", _L), ("W", _I), ("bigram", _P), ("buckets", _L),
+                ("mul_prev", _L), ("mul_cur", _L), ("prev_token", _P), ("out", _P), ("copies", _I), ("n", _L)]
+
+
+class Streams(ctypes.Structure):
+    """Mirror of i64h_streams_args (include/i64h_dense.h)."""
+    _fields_ = [("streams", _P), ("S", _I), ("n", _L), ("W", _I), ("y", _P), ("ldy", _L), ("y2", _P), ("ldy2", _L), ("yn_w", _P), ("y2n_w", _P),
+                ("y_eps", _F), ("mix", _P), ("out_w", _P), ("in_w", _P), ("norm_w", _P), ("norm_w_len", _I), ("eps", _F), ("h", _P), ("rows", _P),
+                ("m_rows", _L)]
+
+
+class CausalConv(ctypes.Structure):
+    """Mirror of i64h_causal_conv_args (include/i64h_dense.h)."""
+    _fields_ = [("P", _P), ("ldp", _L), ("off", _I), ("channels", _I), ("taps", _I), ("w", _P), ("bias", _P), ("positions", _P), ("slot_ids", _P),
+                ("state", _P), ("out", _P), ("ldo", _L), ("n", _L)]
+
+
+class SsmScan(ctypes.Structure):
+    """Mirror of i64h_ssm_scan_args (include/i64h_dense.h)."""
+    _fields_ = [("xbc", _P), ("ldx", _L), ("dt", _P), ("lddt", _L), ("dt_bias", _P), ("A_log", _P), ("Dskip", _P), ("heads", _I), ("vdim", _I),
+                ("state", _I), ("groups", _I), ("seg_start", _P), ("nseg", _I), ("positions", _P), ("slot_ids", _P), ("ssm_state", _P), ("y", _P),
+                ("ldy", _L), ("n", _L)]
+
+
+class GateNorm(ctypes.Structure):
+    """Mirror of i64h_gate_norm_args (include/i64h_dense.h)."""
+    _fields_ = [("y", _P), ("ldy", _L), ("z", _P), ("ldz", _L), ("w", _P), ("width", _I), ("groups", _I), ("eps", _F), ("out", _P), ("ldo", _L), ("n", _L)]
+
+
+class MinGruScan(ctypes.Structure):
+    """Mirror of i64h_mingru_scan_args (include/i64h_dense.h)."""
+    _fields_ = [("P", _P), ("ldp", _L), ("z_off", _I), ("x_off", _I), ("g_off", _I), ("width", _I), ("seg_start", _P), ("nseg", _I), ("positions", _P),
+                ("slot_ids", _P), ("state", _P), ("out", _P), ("ldo", _L), ("n", _L)]
+
+
+class KAttnPrep(ctypes.Structure):
+    """Mirror of i64h_kattn_prep_args (include/i64h_dense.h)."""
+    _fields_ = [("P", _P), ("ldp", _L), ("q_off", _I), ("k_off", _I), ("heads", _I), ("kv_heads", _I), ("dim", _I), ("q_norm_w", _P), ("k_norm_w", _P),
+                ("temp", _P), ("scale", _F), ("eps", _F), ("positions", _P), ("slot_ids", _P), ("block_table", _P), ("max_blocks_per_seq", _I),
+                ("block_size", _I), ("cache", _P), ("cache_dtype", _I), ("kscale", _P), ("Q", _P), ("n", _L)]
+
+
+class KAttn(ctypes.Structure):
+    """Mirror of i64h_kattn_args (include/i64h_dense.h)."""
+    _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("kscale", _P), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
+                ("slot_ids", _P), ("positions", _P), ("chunk", _I), ("bias", _P), ("bias_rows", _I), ("sink", _I), ("out", _P), ("n", _L), ("heads", _I),
+                ("kv_heads", _I), ("dim", _I)]
 
 
 _dense: Optional[ctypes.CDLL] = None

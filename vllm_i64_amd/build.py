@@ -1,7 +1,8 @@
 """Build the in-tree HIP libraries (gfx950 code objects + C ABI) with hipcc.  No GPU needed: hipcc cross-compiles.
 
 libi64hip.so        the quantized token-routed-MoE forward (include/i64h.h)
-libi64hip_dense.so  models with bf16 weights and a 32-bit residual: Linear, gated post-norm, latent attention, sampling
+libi64hip_dense.so  models with bf16 weights and a 32-bit residual: Linear, gated post-norm, latent attention, multi-stream
+                    residual, state-space / gated recurrences, key-valued chunked attention, sampling
                     (include/i64h_dense.h) - a library of its own, so that serving such a model builds nothing else
 """
 from __future__ import annotations
@@ -15,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libi64hip.so")
 DENSE_OUT = os.path.join(HERE, "libi64hip_dense.so")
-DENSE_SOURCES = ["i64h_api.hip", "i64h_dense.hip", "i64h_latent.hip"]
+DENSE_SOURCES = ["i64h_api.hip", "i64h_dense.hip", "i64h_latent.hip", "i64h_hybrid.hip"]
 SOURCES = ["i64h_api.hip", "i64h_route.hip", "i64h_quant.hip", "i64h_norm.hip", "i64h_gemm.hip", "i64h_gemm_os.hip", "i64h_attn.hip", "i64h_moe.hip", "i64h_fp8.hip", "i64h_kv.hip", "i64h_decode.hip", "i64h_variants.hip", "i64h_group_f32.hip", "i64h_lmhead.hip"]
 # -ffp-contract=off: a*b+c stays two roundings unless the source says fmaf, so fp32 element-wise math has the
 # same rounding steps as the reference's CPU ops.
@@ -35,7 +36,8 @@ def _stale(obj: str, src: str) -> bool:
         return True
     t = os.path.getmtime(obj)
     # every object depends on both headers: the public one carries structs that cross translation units
-    deps = [src, os.path.join(os.path.dirname(HERE), "include", "i64h.h"), os.path.abspath(__file__)]
+    inc = os.path.join(os.path.dirname(HERE), "include")
+    deps = [src, os.path.join(inc, "i64h.h"), os.path.join(inc, "i64h_dense.h"), os.path.abspath(__file__)]
     deps += [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     return any(os.path.getmtime(d) > t for d in deps)
 

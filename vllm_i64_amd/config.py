@@ -124,14 +124,108 @@ class DenseMlpConfig:
         return cls(ff=int(m["ff"]))
 
 
-MIXERS = {"latent_attention": LatentAttentionConfig}
+@dataclass
+class Mamba2Config:
+    """State-space mixer with a scalar decay per head: inner = heads * vdim channels, a (state x vdim) matrix per head and sequence,
+    `groups` shared input / output maps, a causal convolution of `conv` taps in front, an RMS norm in `norm_groups` parts behind."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int = 1
+    conv: int = 4
+    norm_groups: int = 1
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+    @property
+    def in_width(self) -> int:
+        return 2 * self.inner + 2 * self.groups * self.state + self.heads
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "Mamba2Config":
+        c = cls(heads=int(m["heads"]), vdim=int(m["vdim"]), state=int(m["state"]), groups=int(m.get("groups", 1)), conv=int(m.get("conv", 1)),
+                norm_groups=int(m.get("norm_groups", 1)))
+        if min(c.heads, c.vdim, c.state, c.groups, c.conv, c.norm_groups) <= 0 or c.heads % c.groups or c.inner % c.norm_groups:
+            raise ValueError(f"mamba2: bad sizes {m}")
+        return c
+
+    def to_dict(self) -> dict:
+        return {"heads": self.heads, "vdim": self.vdim, "state": self.state, "groups": self.groups, "conv": self.conv, "norm_groups": self.norm_groups}
+
+
+@dataclass
+class KeyAttentionConfig:
+    """Attention whose values are the projected keys: whole-row query / key norms, a per-head temperature, a learned bias by bucketed
+    distance (as many buckets as the table has rows, logarithmic up to bias_max), visibility limited to the query's chunk of `chunk`
+    positions (0: all earlier positions), a softmax with one added to the denominator."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    chunk: int = 0
+    bias_max: float = 0.0
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "KeyAttentionConfig":
+        c = cls(heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m.get("vdim", m["dim"])),
+                scale=float(m["scale"]), chunk=int((m.get("mask") or {}).get("size", 0)), bias_max=float(m.get("bias_max", 0.0)))
+        if min(c.heads, c.kv_heads, c.dim) <= 0 or c.heads % c.kv_heads or c.chunk < 0:
+            raise ValueError(f"attention: bad sizes {m}")
+        if c.vdim != c.dim:
+            raise ValueError(f"attention: the values are the keys, so vdim {c.vdim} has to equal dim {c.dim}")
+        return c
+
+    def to_dict(self) -> dict:
+        d = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale, "bias_max": self.bias_max}
+        if self.chunk:
+            d["mask"] = {"size": self.chunk}
+        return d
+
+
+@dataclass
+class MinGruConfig:
+    width: int
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "MinGruConfig":
+        if int(m["width"]) <= 0:
+            raise ValueError(f"gated recurrence: bad width {m}")
+        return cls(width=int(m["width"]))
+
+    def to_dict(self) -> dict:
+        return {"width": self.width}
+
+
+@dataclass
+class ParallelMixerConfig:
+    """Two mixers that read the same input; the result is the mean of their separately normed outputs."""
+    left: KeyAttentionConfig
+    right: MinGruConfig
+
+    @classmethod
+    def from_dict(cls, m: dict) -> "ParallelMixerConfig":
+        return cls(left=KeyAttentionConfig.from_dict(m["left"]), right=MinGruConfig.from_dict(m["right"]))
+
+    def to_dict(self) -> dict:
+        return {"left": self.left.to_dict(), "right": self.right.to_dict()}
+
+
+MIXERS = {"latent_attention": LatentAttentionConfig, "mamba2": Mamba2Config, "parallel": ParallelMixerConfig}
 
 
 @dataclass
 class DecoderLayerConfig:
     type: str
-    mixer: LatentAttentionConfig
+    mixer: object
     mlp: "DenseMlpConfig | None"
+    weights_of: "int | None" = None      # the layer whose tensors this layer uses (its cache and state stay its own)
 
     @classmethod
     def from_dict(cls, d: dict) -> "DecoderLayerConfig":
@@ -139,7 +233,9 @@ class DecoderLayerConfig:
         if kind not in MIXERS:
             raise ValueError(f"layer type '{kind}' is not built (known: {sorted(MIXERS)})")
         mlp = d.get("mlp")
-        return cls(type=kind, mixer=MIXERS[kind].from_dict(d["mixer"]), mlp=DenseMlpConfig.from_dict(mlp) if mlp else None)
+        share = d.get("weights_of")
+        return cls(type=kind, mixer=MIXERS[kind].from_dict(d["mixer"]), mlp=DenseMlpConfig.from_dict(mlp) if mlp else None,
+                   weights_of=int(share) if share is not None else None)
 
 
 @dataclass
@@ -189,3 +285,76 @@ class MorilornConfig:
             layers.append({"type": l.type, "mixer": mixer, "mlp": {"kind": "dense", "ff": l.mlp.ff} if l.mlp else None})
         return {"architecture": "Morilorn", "vocab": self.vocab, "width": self.width, "layers": layers, "embedding": {"scale": self.embedding_scale},
                 "postln_alpha": self.postln_alpha, "norm": {"eps": self.norm_eps, "groups": self.norm_groups}, "logit_softcap": self.logit_softcap}
+
+
+# ---------------------------------------------------------------------------------------------------------------------------
+# Dogalorn: pre-norm decoder with a multi-stream residual (hyper-connections), single-number RMS norm weights, a hashed bigram
+# embedding, layers that may borrow another layer's tensors, and two kinds of mixer: a state-space layer, and an attention over
+# chunks of positions side by side with a gated recurrence.  Every size and constant comes from the checkpoint's config.json.
+# ---------------------------------------------------------------------------------------------------------------------------
+@dataclass
+class BigramConfig:
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+
+
+@dataclass
+class DogalornConfig:
+    vocab: int
+    width: int
+    layers: list
+    norm_eps: float = 1e-6
+    streams: int = 0               # 0: the ordinary residual sum
+    logit_scale: float = 1.0
+    bigram: "BigramConfig | None" = None
+    name: str = "Dogalorn"
+
+    LAYER_TYPES = ("mamba2", "parallel")
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
+    @property
+    def max_pos(self) -> int:
+        """Positions are computed, not tabulated: a sequence is bounded by the page pool only."""
+        return 1 << 30
+
+    @classmethod
+    def from_dict(cls, d: dict) -> "DogalornConfig":
+        bg = (d.get("embedding") or {}).get("bigram")
+        layers = [DecoderLayerConfig.from_dict(l) for l in d["layers"]]
+        c = cls(vocab=int(d["vocab"]), width=int(d["width"]), layers=layers, norm_eps=float((d.get("norm") or {}).get("eps", 1e-6)),
+                streams=int(d.get("streams") or 0), logit_scale=float(d.get("logit_scale", 1.0)),
+                bigram=BigramConfig(int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"])) if bg else None,
+                name=str(d.get("architecture", "Dogalorn")))
+        for i, l in enumerate(layers):
+            if l.type not in cls.LAYER_TYPES:
+                raise ValueError(f"layer {i}: type '{l.type}' is not part of this design (known: {cls.LAYER_TYPES})")
+            if l.weights_of is not None:
+                j = l.weights_of
+                if not 0 <= j < len(layers) or layers[j].weights_of is not None or (layers[j].type, layers[j].mixer, layers[j].mlp) != (l.type, l.mixer, l.mlp):
+                    raise ValueError(f"layer {i}: borrows the tensors of layer {j}, which is no layer of the same shape with tensors of its own")
+        if c.bigram is not None and c.bigram.buckets <= 0:
+            raise ValueError("bigram embedding: no buckets")
+        return c
+
+    def to_dict(self) -> dict:
+        layers = []
+        for l in self.layers:
+            e = {"type": l.type, "mixer": l.mixer.to_dict(), "mlp": {"kind": "dense", "ff": l.mlp.ff} if l.mlp else None}
+            if l.weights_of is not None:
+                e["weights_of"] = l.weights_of
+            layers.append(e)
+        d = {"architecture": "Dogalorn", "vocab": self.vocab, "width": self.width, "layers": layers, "norm": {"eps": self.norm_eps},
+             "logit_scale": self.logit_scale}
+        if self.streams:
+            d["streams"] = self.streams
+        if self.bigram is not None:
+            d["embedding"] = {"bigram": {"buckets": self.bigram.buckets, "mul_prev": self.bigram.mul_prev, "mul_cur": self.bigram.mul_cur}}
+        return d

@@ -29,9 +29,14 @@ __device__ __forceinline__ float dn_gelu_tanh(float z) {
     return 0.5f * z * (1.0f + tanhf(inner));
 }
 
+__device__ __forceinline__ float dn_gelu_erf(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
+
 template <int EPI>
 __device__ __forceinline__ float dn_epilogue(const i64h_linear& p, float acc, float acc2, int64_t b, int64_t r, int c) {
     if (EPI == I64H_EPI_GELU_MUL) return dn_gelu_tanh(acc) * acc2;
+    if (p.bias) acc += p.bias[b * p.bias_batch + c];
+    if (EPI == I64H_EPI_GELU_ERF) return dn_gelu_erf(acc);
+    if (EPI == I64H_EPI_SCALE) return acc * p.scale;
     if (EPI == I64H_EPI_MUL_SIGMOID) return acc * dn_sigmoid(p.E[b * p.e_batch + r * p.lde + c]);
     if (EPI == I64H_EPI_SOFTCAP) return p.softcap * tanhf(acc / p.softcap);
     return acc;
@@ -659,6 +664,8 @@ static void launch_tile(const i64h_linear& d, dim3 grid, hipStream_t s, int vecA
         case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_GELU_MUL>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_MUL_SIGMOID>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+        case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_GELU_ERF>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+        case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_SCALE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         default: hipLaunchKernelGGL((linear_tile_kernel<EXACT, I64H_EPI_STORE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
     }
 }
@@ -684,9 +691,10 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
     const i64h_linear& d = *dp;
     I64H_CHECK_ARG(d.M >= 0 && d.N > 0 && d.K > 0 && d.batch > 0, "linear: bad sizes M=%lld N=%d K=%d batch=%d", (long long)d.M, d.N, d.K, d.batch);
     I64H_CHECK_ARG(d.A && d.W && d.C, "linear: null operand");
-    I64H_CHECK_ARG(d.epilogue >= 0 && d.epilogue <= 3, "linear: epilogue %d", d.epilogue);
+    I64H_CHECK_ARG(d.epilogue >= 0 && d.epilogue <= 5, "linear: epilogue %d", d.epilogue);
     I64H_CHECK_ARG(d.epilogue != I64H_EPI_MUL_SIGMOID || d.E, "linear: the sigmoid epilogue needs E");
     I64H_CHECK_ARG(d.epilogue != I64H_EPI_SOFTCAP || d.softcap > 0.0f, "linear: soft cap %g", (double)d.softcap);
+    I64H_CHECK_ARG(d.epilogue != I64H_EPI_GELU_MUL || !d.bias, "linear: the gate / up epilogue takes no bias");
     I64H_CHECK_ARG(d.lda >= d.K || d.M <= 1, "linear: lda %lld < K %d", (long long)d.lda, d.K);
     I64H_CHECK_ARG(d.batch <= 65535 && (d.M + 63) / 64 <= 65535, "linear: grid too large");
     if (d.M == 0) return 0;
@@ -702,6 +710,8 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
             case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_GELU_MUL>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), lds, s, d, cpb); break;
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), lds, s, d, cpb); break;
+            case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_GELU_ERF>), grid, dim3(256), lds, s, d, cpb); break;
+            case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_SCALE>), grid, dim3(256), lds, s, d, cpb); break;
             default: hipLaunchKernelGGL((linear_skinny_kernel<I64H_EPI_STORE>), grid, dim3(256), lds, s, d, cpb); break;
         }
         I64H_CHECK_LAUNCH();
@@ -714,6 +724,8 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
             case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_GELU_MUL, 4>), grid, dim3(256), 0, s, d); break;
             case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_MUL_SIGMOID, 8>), grid, dim3(512), 0, s, d); break;
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SOFTCAP, 8>), grid, dim3(512), 0, s, d); break;
+            case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_GELU_ERF, 8>), grid, dim3(512), 0, s, d); break;
+            case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_SCALE, 8>), grid, dim3(512), 0, s, d); break;
             default: hipLaunchKernelGGL((linear_rows64_kernel<I64H_EPI_STORE, 8>), grid, dim3(512), 0, s, d); break;
         }
         I64H_CHECK_LAUNCH();
@@ -726,6 +738,8 @@ int i64h_linear_run(const i64h_linear* dp, void* stream) {
             case I64H_EPI_GELU_MUL: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_GELU_MUL>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_MUL_SIGMOID: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_MUL_SIGMOID>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             case I64H_EPI_SOFTCAP: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_SOFTCAP>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+            case I64H_EPI_GELU_ERF: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_GELU_ERF>), grid, dim3(256), 0, s, d, vecA, vecW); break;
+            case I64H_EPI_SCALE: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_SCALE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
             default: hipLaunchKernelGGL((linear_tile128_kernel<I64H_EPI_STORE>), grid, dim3(256), 0, s, d, vecA, vecW); break;
         }
         I64H_CHECK_LAUNCH();

@@ -1,0 +1,485 @@
+// Kernels of libi64hip_dense.so for recurrent and hybrid layers (include/i64h_dense.h, "recurrent and hybrid layers"):
+//   embed_bigram_kernel / prev_token_kernel : token embedding + hashed bigram embedding; the previous token is per-sequence state
+//   streams_kernel        : multi-stream residual write + the next sublayer's weighted read and RMS norm, one workgroup per row
+//   causal_conv_kernel / conv_carry_kernel : per-channel causal convolution + silu over rows and carried inputs; the carry update
+//   ssm_scan_kernel       : state-space recurrence with a scalar decay per head, the (state x vdim) matrix of a head in LDS
+//   gate_norm_kernel      : y * silu(z) -> RMS norm in groups
+//   mingru_scan_kernel    : element-wise gated recurrence
+//   kattn_prep_kernel     : whole-row RMS norms of query and key, key-norm weights / scale / temperature folded into the query,
+//                           raw key row and its 1 / rms into the paged cache
+//   kattn_row_kernel      : attention over the cached keys (which are also the values) with distance bias, chunk mask and sink
+// A row continues the row before it iff slot and position say so; state is taken as empty at position 0.  All arithmetic fp32.
+#include "i64h_common.h"
+#include "i64h_dense.h"
+
+__device__ __forceinline__ float hy_bf16(const void* p, int64_t i) { return __uint_as_float((uint32_t)((const uint16_t*)p)[i] << 16); }
+__device__ __forceinline__ float hy_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float hy_silu(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float hy_softplus(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
+__device__ __forceinline__ bool hy_continues(const int32_t* slot, const int32_t* pos, int64_t t, int d) {
+    // row t - d belongs to the same run of consecutive positions as row t
+    return t - d >= 0 && slot[t - d] == slot[t] && pos[t - d] == pos[t] - d;
+}
+
+// sum over the 256 threads of a workgroup; red: 4 floats of LDS
+__device__ __forceinline__ float hy_block_sum(float v, float* red) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void embed_bigram_kernel(const i64h_embed_bigram_args p) {
+    const int64_t t = blockIdx.x;
+    int64_t id = p.ids[t];
+    id = id < 0 ? 0 : (id >= p.V ? p.V - 1 : id);
+    const int W = p.W;
+    int64_t brow = -1;
+    if (p.bigram) {
+        if (p.positions[t] == 0) brow = p.buckets;
+        else {
+            int64_t prev = hy_continues(p.slot_ids, p.positions, t, 1) ? p.ids[t - 1] : p.prev_token[p.slot_ids[t]];
+            prev = prev < 0 ? 0 : (prev >= p.V ? p.V - 1 : prev);
+            brow = (prev * p.mul_prev + id * p.mul_cur) % p.buckets;
+        }
+    }
+    const int64_t plane = p.n * (int64_t)W;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float v = hy_bf16(p.table, id * W + c);
+        if (brow >= 0) v += hy_bf16(p.bigram, brow * W + c);
+        for (int s = 0; s < p.copies; ++s) p.out[s * plane + t * W + c] = v;
+    }
+}
+
+__global__ __launch_bounds__(256) void prev_token_kernel(const i64h_embed_bigram_args p) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= p.n) return;
+    if (t + 1 < p.n && hy_continues(p.slot_ids, p.positions, t + 1, 1)) return;   // not the last row of its run
+    p.prev_token[p.slot_ids[t]] = p.ids[t];
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+#define HY_MAX_STREAMS 8
+__global__ __launch_bounds__(256) void streams_kernel(const i64h_streams_args p) {
+    extern __shared__ float sv[];   // [W] the weighted read of the row, then 4 floats for reductions
+    const int tid = threadIdx.x;
+    const int W = p.W, S = p.S;
+    float* red = sv + W;
+    const int64_t m = blockIdx.x;
+    const int64_t r = p.rows ? (int64_t)p.rows[m] : m;
+    const int64_t plane = p.n * (int64_t)W;
+    float* xs = p.streams + r * W;
+    float ya = 1.0f, yb = 1.0f;
+    if (p.y && p.y2) {   // the two side-by-side results, each divided by its root mean square
+        float a = 0.0f, b = 0.0f;
+        for (int c = tid; c < W; c += 256) {
+            const float u = p.y[m * p.ldy + c], v = p.y2[m * p.ldy2 + c];
+            a += u * u;
+            b += v * v;
+        }
+        a = hy_block_sum(a, red);
+        b = hy_block_sum(b, red);
+        ya = 1.0f / sqrtf(a / (float)W + p.y_eps);
+        yb = 1.0f / sqrtf(b / (float)W + p.y_eps);
+    }
+    float ss = 0.0f;
+    for (int c = tid; c < W; c += 256) {
+        float x[HY_MAX_STREAMS];
+#pragma unroll
+        for (int s = 0; s < HY_MAX_STREAMS; ++s) x[s] = s < S ? xs[s * plane + c] : 0.0f;
+        if (p.y) {
+            float v = p.y[m * p.ldy + c];
+            if (p.y2) v = 0.5f * (v * ya * p.yn_w[c] + p.y2[m * p.ldy2 + c] * yb * p.y2n_w[c]);
+            float nx[HY_MAX_STREAMS];
+#pragma unroll
+            for (int t = 0; t < HY_MAX_STREAMS; ++t) {
+                float a = 0.0f;
+                if (t < S) {
+                    if (p.mix) {
+#pragma unroll
+                        for (int s = 0; s < HY_MAX_STREAMS; ++s)
+                            if (s < S) a += p.mix[s * S + t] * x[s];
+                    } else a = x[t];
+                    a += p.out_w[t] * v;
+                    xs[t * plane + c] = a;
+                }
+                nx[t] = a;
+            }
+#pragma unroll
+            for (int t = 0; t < HY_MAX_STREAMS; ++t) x[t] = nx[t];
+        }
+        if (p.h) {
+            float u = 0.0f;
+#pragma unroll
+            for (int s = 0; s < HY_MAX_STREAMS; ++s)
+                if (s < S) u += (p.in_w ? p.in_w[s] : 1.0f) * x[s];
+            sv[c] = u;
+            ss += u * u;
+        }
+    }
+    if (!p.h) return;
+    ss = hy_block_sum(ss, red);
+    const float den = sqrtf(ss / (float)W + p.eps);
+    for (int c = tid; c < W; c += 256) p.h[m * W + c] = sv[c] / den * p.norm_w[p.norm_w_len == 1 ? 0 : c];
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// the input of channel c, d positions before row t (d >= 1); `before` = rows of this step that continue into row t (at most taps - 1 counted)
+__device__ __forceinline__ float conv_input(const i64h_causal_conv_args& p, int64_t t, int d, int before, int c) {
+    if (p.positions[t] - d < 0) return 0.0f;
+    if (d <= before) return p.P[(t - d) * p.ldp + p.off + c];
+    return p.state[((int64_t)p.slot_ids[t] * (p.taps - 1) + (p.taps - 1 + before - d)) * p.channels + c];
+}
+__device__ __forceinline__ int conv_rows_before(const i64h_causal_conv_args& p, int64_t t) {
+    int before = 0;
+    while (before < p.taps - 1 && hy_continues(p.slot_ids, p.positions, t, before + 1)) ++before;
+    return before;
+}
+
+__global__ __launch_bounds__(256) void causal_conv_kernel(const i64h_causal_conv_args p) {
+    const int64_t t = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= p.channels) return;
+    const int before = conv_rows_before(p, t);
+    float a = p.bias ? p.bias[c] : 0.0f;
+    for (int k = 0; k < p.taps - 1; ++k) a += p.w[(int64_t)c * p.taps + k] * conv_input(p, t, p.taps - 1 - k, before, c);
+    a += p.w[(int64_t)c * p.taps + p.taps - 1] * p.P[t * p.ldp + p.off + c];
+    p.out[t * p.ldo + c] = hy_silu(a);
+}
+
+#define HY_MAX_TAPS 16
+__global__ __launch_bounds__(256) void conv_carry_kernel(const i64h_causal_conv_args p) {
+    const int64_t t = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (t + 1 < p.n && hy_continues(p.slot_ids, p.positions, t + 1, 1)) return;   // only the last row of a run
+    if (c >= p.channels) return;
+    const int before = conv_rows_before(p, t);
+    float v[HY_MAX_TAPS];   // the inputs 0 .. taps - 2 positions back, read before any is overwritten
+    for (int d = 0; d < p.taps - 1; ++d) v[d] = d == 0 ? p.P[t * p.ldp + p.off + c] : conv_input(p, t, d, before, c);
+    for (int d = 0; d < p.taps - 1; ++d) p.state[((int64_t)p.slot_ids[t] * (p.taps - 1) + (p.taps - 2 - d)) * p.channels + c] = v[d];
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+// one workgroup per (head, run of rows): thread (lane over the state index, value column); the head's matrix stays in LDS
+__global__ __launch_bounds__(256) void ssm_scan_kernel(const i64h_ssm_scan_args p) {
+    extern __shared__ float sm[];
+    const int N = p.state, P = p.vdim;
+    const int nl = 256 / P;                  // threads per value column
+    float* sS = sm;                          // [N, P]
+    float* sB = sS + (int64_t)N * P;         // [N]
+    float* sC = sB + N;                      // [N]
+    float* sX = sC + N;                      // [P]
+    float* sY = sX + P;                      // [nl, P]
+    const int tid = threadIdx.x;
+    const int a = blockIdx.x, seg = blockIdx.y;
+    const int g = a / (p.heads / p.groups);
+    const int64_t r0 = p.seg_start[seg], r1 = p.seg_start[seg + 1];
+    if (r1 <= r0) return;
+    const int slot = p.slot_ids[r0];
+    float* gS = p.ssm_state + ((int64_t)slot * p.heads + a) * N * P;
+    const bool fresh = p.positions[r0] == 0;
+    for (int i = tid; i < N * P; i += 256) sS[i] = fresh ? 0.0f : gS[i];
+    const int col = tid % P, nlane = tid / P;
+    const bool active = nlane < nl;
+    const float dtb = p.dt_bias[a], Aneg = -expf(p.A_log[a]), Dk = p.Dskip[a];
+    const int inner = p.heads * P;
+    __syncthreads();
+    for (int64_t t = r0; t < r1; ++t) {
+        const float* row = p.xbc + t * p.ldx;
+        for (int i = tid; i < N; i += 256) {
+            sB[i] = row[inner + g * N + i];
+            sC[i] = row[inner + (p.groups + g) * N + i];
+        }
+        if (tid < P) sX[tid] = row[a * P + tid];
+        const float dt = hy_softplus(p.dt[t * p.lddt + a] + dtb);
+        const float decay = expf(Aneg * dt);
+        __syncthreads();
+        if (active) {
+            const float xv = dt * sX[col];
+            float part = 0.0f;
+            for (int n = nlane; n < N; n += nl) {
+                const float s = decay * sS[n * P + col] + sB[n] * xv;
+                sS[n * P + col] = s;
+                part += s * sC[n];
+            }
+            sY[nlane * P + col] = part;
+        }
+        __syncthreads();
+        if (tid < P) {
+            float y = 0.0f;
+            for (int i = 0; i < nl; ++i) y += sY[i * P + tid];
+            p.y[t * p.ldy + a * P + tid] = y + Dk * sX[tid];
+        }
+        __syncthreads();
+    }
+    for (int i = tid; i < N * P; i += 256) gS[i] = sS[i];
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gate_norm_kernel(const i64h_gate_norm_args p) {
+    extern __shared__ float sv[];   // [width] gated values, [groups] root mean squares
+    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
+    const int64_t m = blockIdx.x;
+    const int W = p.width;
+    for (int c = tid; c < W; c += 256) {
+        float v = p.y[m * p.ldy + c];
+        if (p.z) v *= hy_silu(p.z[m * p.ldz + c]);
+        sv[c] = v;
+    }
+    __syncthreads();
+    const int gs = W / p.groups;
+    for (int g = wid; g < p.groups; g += 4) {
+        float s = 0.0f;
+        for (int c = lane; c < gs; c += 64) {
+            const float v = sv[g * gs + c];
+            s += v * v;
+        }
+        s = wave_sum(s);
+        if (lane == 0) sv[W + g] = sqrtf(s / (float)gs + p.eps);
+    }
+    __syncthreads();
+    for (int c = tid; c < W; c += 256) p.out[m * p.ldo + c] = sv[c] / sv[W + c / gs] * p.w[c];
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void mingru_scan_kernel(const i64h_mingru_scan_args p) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    const int seg = blockIdx.y;
+    if (c >= p.width) return;
+    const int64_t r0 = p.seg_start[seg], r1 = p.seg_start[seg + 1];
+    if (r1 <= r0) return;
+    float* st = p.state + (int64_t)p.slot_ids[r0] * p.width + c;
+    float S = p.positions[r0] == 0 ? 0.0f : *st;
+    for (int64_t t = r0; t < r1; ++t) {
+        const float* row = p.P + t * p.ldp;
+        const float z = hy_sigmoid(row[p.z_off + c]);
+        const float u = row[p.x_off + c];
+        const float cand = u >= 0.0f ? u + 0.5f : hy_sigmoid(u);
+        S = (1.0f - z) * S + z * cand;
+        p.out[t * p.ldo + c] = S * hy_silu(row[p.g_off + c]);
+    }
+    *st = S;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int64_t cache_row(const int32_t* bt, int mbs, int bs, int slot, int pos) {
+    return (int64_t)bt[(int64_t)slot * mbs + pos / bs] * bs + pos % bs;
+}
+
+__global__ __launch_bounds__(256) void kattn_prep_kernel(const i64h_kattn_prep_args p) {
+    __shared__ float red[4];
+    const int tid = threadIdx.x;
+    const int64_t t = blockIdx.x;
+    const int nq = p.heads * p.dim, nk = p.kv_heads * p.dim;
+    const float* q = p.P + t * p.ldp + p.q_off;
+    const float* k = p.P + t * p.ldp + p.k_off;
+    float a = 0.0f, b = 0.0f;
+    for (int c = tid; c < nq; c += 256) a += q[c] * q[c];
+    for (int c = tid; c < nk; c += 256) b += k[c] * k[c];
+    a = hy_block_sum(a, red);
+    b = hy_block_sum(b, red);
+    const float qr = 1.0f / sqrtf(a / (float)nq + p.eps);
+    const float kr = 1.0f / sqrtf(b / (float)nk + p.eps);
+    const int rep = p.heads / p.kv_heads;
+    for (int c = tid; c < nq; c += 256) {
+        const int h = c / p.dim, d = c % p.dim;
+        float v = q[c] * qr * p.q_norm_w[c] * p.k_norm_w[(h / rep) * p.dim + d] * p.scale;
+        if (p.temp) v *= p.temp[h];
+        p.Q[t * nq + c] = v;
+    }
+    const int64_t row = cache_row(p.block_table, p.max_blocks_per_seq, p.block_size, p.slot_ids[t], p.positions[t]);
+    if (p.cache_dtype == 0) {
+        float* dst = (float*)p.cache + row * nk;
+        for (int c = tid; c < nk; c += 256) dst[c] = k[c];
+    } else {
+        __bf16* dst = (__bf16*)p.cache + row * nk;
+        for (int c = tid; c < nk; c += 256) dst[c] = (__bf16)k[c];
+    }
+    if (tid == 0) p.kscale[row] = kr;
+}
+
+// one wave per (row, head): the lanes take 64 keys at a time for the scores, then the value columns for the weighted sum
+#define KA_MAX_DIM 256
+template <typename T>
+__global__ __launch_bounds__(256) void kattn_row_kernel(const i64h_kattn_args p) {
+    __shared__ float sq[4][KA_MAX_DIM];
+    __shared__ float sp[4][64];
+    __shared__ int64_t srow[4][64];
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int64_t item = (int64_t)blockIdx.x * 4 + wid;
+    if (item >= p.n * p.heads) return;     // (a whole wave leaves; no workgroup barrier below)
+    const int64_t t = item / p.heads;
+    const int h = (int)(item % p.heads);
+    const int g = h / (p.heads / p.kv_heads);
+    const int dim = p.dim, nk = p.kv_heads * dim;
+    const int pos = p.positions[t], slot = p.slot_ids[t];
+    const int lo = p.chunk > 0 ? (pos / p.chunk) * p.chunk : 0;
+    const T* cache = (const T*)p.cache;
+    for (int d = lane; d < dim; d += 64) sq[wid][d] = p.Q[(t * p.heads + h) * dim + d];
+    float m = p.sink ? 0.0f : -INFINITY, l = p.sink ? 1.0f : 0.0f;
+    float acc[KA_MAX_DIM / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int j0 = lo; j0 <= pos; j0 += 64) {
+        const int j = j0 + lane;
+        float s = -INFINITY;
+        int64_t row = 0;
+        if (j <= pos) {
+            row = cache_row(p.block_table, p.max_blocks_per_seq, p.block_size, slot, j);
+            const T* kr = cache + row * nk + g * dim;
+            float dot = 0.0f;
+            for (int d = 0; d < dim; ++d) dot += sq[wid][d] * (float)kr[d];
+            s = dot * p.kscale[row];
+            if (p.bias) s += p.bias[(int64_t)min(pos - j, p.bias_rows - 1) * p.heads + h];
+        }
+        srow[wid][lane] = row;
+        const float mn = fmaxf(m, wave_max(s));
+        const float w = j <= pos ? expf(s - mn) : 0.0f;
+        const float f = expf(m - mn);      // m is finite or the first tile has a key (mn finite): no inf - inf
+        l = l * f + wave_sum(w);
+        m = mn;
+        sp[wid][lane] = w;
+        const int cnt = min(64, pos - j0 + 1);
+#pragma unroll
+        for (int i = 0; i < KA_MAX_DIM / 64; ++i) {
+            const int d = lane + 64 * i;
+            if (d < dim) {
+                float a = acc[i] * f;
+                for (int u = 0; u < cnt; ++u) a += sp[wid][u] * (float)cache[srow[wid][u] * nk + g * dim + d];
+                acc[i] = a;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < KA_MAX_DIM / 64; ++i) {
+        const int d = lane + 64 * i;
+        if (d < dim) p.out[(t * p.heads + h) * dim + d] = acc[i] / l;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------------
+extern "C" {
+
+int i64h_embed_bigram(const i64h_embed_bigram_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "embed_bigram: no descriptor");
+    const i64h_embed_bigram_args& d = *dp;
+    I64H_CHECK_ARG(d.n >= 0 && d.W > 0 && d.V > 0 && d.copies >= 1, "embed_bigram: bad sizes");
+    I64H_CHECK_ARG(d.ids && d.table && d.out && d.positions && d.slot_ids, "embed_bigram: null operand");
+    I64H_CHECK_ARG(!d.bigram || (d.buckets > 0 && d.prev_token), "embed_bigram: the bigram table needs buckets and the previous tokens");
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(embed_bigram_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    if (d.bigram) {
+        hipLaunchKernelGGL(prev_token_kernel, dim3((unsigned)((d.n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, d);
+        I64H_CHECK_LAUNCH();
+    }
+    return 0;
+}
+
+int i64h_streams_step(const i64h_streams_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "streams: no descriptor");
+    const i64h_streams_args& d = *dp;
+    I64H_CHECK_ARG(d.S >= 1 && d.S <= HY_MAX_STREAMS && d.W > 0 && d.n >= 0, "streams: %d streams (at most %d), width %d", d.S, HY_MAX_STREAMS, d.W);
+    I64H_CHECK_ARG(d.streams && (d.y || d.h), "streams: nothing to do");
+    I64H_CHECK_ARG(!d.y || d.out_w, "streams: the write needs out_w");
+    I64H_CHECK_ARG(!d.y2 || (d.y && d.yn_w && d.y2n_w), "streams: two results need both norm weights");
+    I64H_CHECK_ARG(!d.h || (d.norm_w && (d.norm_w_len == 1 || d.norm_w_len == d.W)), "streams: the read needs a norm weight of 1 or W values");
+    I64H_CHECK_ARG(!d.rows || !d.y, "streams: gathered rows are read only");
+    const int64_t rows = d.rows ? d.m_rows : d.n;
+    const size_t lds = ((size_t)d.W + 4) * 4;
+    I64H_CHECK_ARG(lds <= 64 * 1024, "streams: a row of %d values does not fit the kernel's LDS buffer", d.W);
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(streams_kernel, dim3((unsigned)rows), dim3(256), lds, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_causal_conv(const i64h_causal_conv_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "causal_conv: no descriptor");
+    const i64h_causal_conv_args& d = *dp;
+    I64H_CHECK_ARG(d.channels > 0 && d.taps >= 1 && d.taps <= HY_MAX_TAPS && d.n >= 0, "causal_conv: %d channels, %d taps (at most %d)", d.channels, d.taps, HY_MAX_TAPS);
+    I64H_CHECK_ARG(d.P && d.w && d.out && d.positions && d.slot_ids && (d.state || d.taps == 1), "causal_conv: null operand");
+    I64H_CHECK_ARG(d.n <= 65535, "causal_conv: %lld rows in one launch (at most 65535)", (long long)d.n);
+    if (d.n == 0) return 0;
+    const dim3 grid((unsigned)((d.channels + 255) / 256), (unsigned)d.n);
+    hipLaunchKernelGGL(causal_conv_kernel, grid, dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    if (d.taps > 1) {
+        hipLaunchKernelGGL(conv_carry_kernel, grid, dim3(256), 0, (hipStream_t)stream, d);
+        I64H_CHECK_LAUNCH();
+    }
+    return 0;
+}
+
+int i64h_ssm_scan(const i64h_ssm_scan_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "ssm_scan: no descriptor");
+    const i64h_ssm_scan_args& d = *dp;
+    I64H_CHECK_ARG(d.heads > 0 && d.vdim > 0 && d.vdim <= 256 && d.state > 0 && d.groups > 0 && d.heads % d.groups == 0,
+                   "ssm_scan: heads %d, groups %d, state %d, vdim %d (at most 256)", d.heads, d.groups, d.state, d.vdim);
+    I64H_CHECK_ARG(d.xbc && d.dt && d.dt_bias && d.A_log && d.Dskip && d.seg_start && d.positions && d.slot_ids && d.ssm_state && d.y, "ssm_scan: null operand");
+    const int nl = 256 / d.vdim;
+    const size_t lds = ((size_t)d.state * d.vdim + 2 * (size_t)d.state + d.vdim + (size_t)nl * d.vdim) * 4;
+    I64H_CHECK_ARG(lds <= 64 * 1024, "ssm_scan: a head's state of %d x %d values does not fit the kernel's LDS buffer", d.state, d.vdim);
+    I64H_CHECK_ARG(d.nseg <= 65535, "ssm_scan: %d runs in one launch", d.nseg);
+    if (d.nseg <= 0 || d.n == 0) return 0;
+    hipLaunchKernelGGL(ssm_scan_kernel, dim3((unsigned)d.heads, (unsigned)d.nseg), dim3(256), lds, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_gate_norm(const i64h_gate_norm_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "gate_norm: no descriptor");
+    const i64h_gate_norm_args& d = *dp;
+    I64H_CHECK_ARG(d.width > 0 && d.groups > 0 && d.width % d.groups == 0, "gate_norm: width %d does not split into %d groups", d.width, d.groups);
+    I64H_CHECK_ARG(d.y && d.w && d.out, "gate_norm: null operand");
+    const size_t lds = ((size_t)d.width + d.groups) * 4;
+    I64H_CHECK_ARG(lds <= 64 * 1024, "gate_norm: a row of %d values does not fit the kernel's LDS buffer", d.width);
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(gate_norm_kernel, dim3((unsigned)d.n), dim3(256), lds, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_mingru_scan(const i64h_mingru_scan_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "mingru_scan: no descriptor");
+    const i64h_mingru_scan_args& d = *dp;
+    I64H_CHECK_ARG(d.width > 0 && d.P && d.seg_start && d.positions && d.slot_ids && d.state && d.out, "mingru_scan: bad arguments");
+    I64H_CHECK_ARG(d.nseg <= 65535, "mingru_scan: %d runs in one launch", d.nseg);
+    if (d.nseg <= 0 || d.n == 0) return 0;
+    hipLaunchKernelGGL(mingru_scan_kernel, dim3((unsigned)((d.width + 255) / 256), (unsigned)d.nseg), dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_kattn_prep(const i64h_kattn_prep_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "kattn_prep: no descriptor");
+    const i64h_kattn_prep_args& d = *dp;
+    I64H_CHECK_ARG(d.heads > 0 && d.kv_heads > 0 && d.heads % d.kv_heads == 0 && d.dim > 0, "kattn_prep: heads %d, kv heads %d, dim %d", d.heads, d.kv_heads, d.dim);
+    I64H_CHECK_ARG(d.P && d.q_norm_w && d.k_norm_w && d.positions && d.slot_ids && d.block_table && d.cache && d.kscale && d.Q, "kattn_prep: null operand");
+    I64H_CHECK_ARG(d.cache_dtype == 0 || d.cache_dtype == 2, "kattn_prep: cache type %d", d.cache_dtype);
+    I64H_CHECK_ARG(d.block_size > 0 && d.max_blocks_per_seq > 0, "kattn_prep: bad paging");
+    if (d.n == 0) return 0;
+    hipLaunchKernelGGL(kattn_prep_kernel, dim3((unsigned)d.n), dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+int i64h_kattn(const i64h_kattn_args* dp, void* stream) {
+    I64H_CHECK_ARG(dp != nullptr, "kattn: no descriptor");
+    const i64h_kattn_args& d = *dp;
+    I64H_CHECK_ARG(d.heads > 0 && d.kv_heads > 0 && d.heads % d.kv_heads == 0 && d.dim > 0 && d.dim <= KA_MAX_DIM, "kattn: heads %d, kv heads %d, dim %d (at most %d)",
+                   d.heads, d.kv_heads, d.dim, KA_MAX_DIM);
+    I64H_CHECK_ARG(d.Q && d.cache && d.kscale && d.block_table && d.slot_ids && d.positions && d.out, "kattn: null operand");
+    I64H_CHECK_ARG(d.cache_dtype == 0 || d.cache_dtype == 2, "kattn: cache type %d", d.cache_dtype);
+    I64H_CHECK_ARG(!d.bias || d.bias_rows > 0, "kattn: an empty bias table");
+    I64H_CHECK_ARG(d.block_size > 0 && d.max_blocks_per_seq > 0, "kattn: bad paging");
+    if (d.n == 0) return 0;
+    const int64_t items = d.n * d.heads;
+    const dim3 grid((unsigned)((items + 3) / 4));
+    if (d.cache_dtype == 0) hipLaunchKernelGGL((kattn_row_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, d);
+    else hipLaunchKernelGGL((kattn_row_kernel<__bf16>), grid, dim3(256), 0, (hipStream_t)stream, d);
+    I64H_CHECK_LAUNCH();
+    return 0;
+}
+
+}  // extern "C"

@@ -11,7 +11,7 @@ from . import _lib
 from ._lib import call_dense, ptr
 from .ops import _chk, _stream
 
-EPI_STORE, EPI_GELU_MUL, EPI_MUL_SIGMOID, EPI_SOFTCAP = 0, 1, 2, 3
+EPI_STORE, EPI_GELU_MUL, EPI_MUL_SIGMOID, EPI_SOFTCAP, EPI_GELU_ERF, EPI_SCALE = 0, 1, 2, 3, 4, 5
 CACHE_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 2}
 
 
@@ -22,10 +22,11 @@ def _ref(s):
 def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, m: Optional[int] = None, n: Optional[int] = None, k: Optional[int] = None,
            a_off: int = 0, lda: Optional[int] = None, a_rows: Optional[torch.Tensor] = None, c_off: int = 0, ldc: Optional[int] = None,
            batch: int = 1, a_batch: int = 0, w_batch: int = 0, c_batch: int = 0, exact: bool = False, epilogue: int = EPI_STORE,
-           e: Optional[torch.Tensor] = None, e_off: int = 0, lde: int = 0, e_batch: int = 0, softcap: float = 0.0) -> torch.Tensor:
+           e: Optional[torch.Tensor] = None, e_off: int = 0, lde: int = 0, e_batch: int = 0, softcap: float = 0.0,
+           bias: Optional[torch.Tensor] = None, bias_batch: int = 0, scale: float = 1.0) -> torch.Tensor:
     """out[b][:, c_off + b * c_batch : + n] = epilogue(a[b][rows, a_off + b * a_batch : + k] @ w[b]^T): see i64h_linear.  a, out and e are
     fp32 matrices addressed by (column offset, row stride); w is bf16 [n, k] (EPI_GELU_MUL: [2n, k], gate rows first), or a stack
-    [batch, n, k] with w_batch = n * k."""
+    [batch, n, k] with w_batch = n * k.  bias fp32 [n] (per batch: bias_batch apart) is added before the epilogue."""
     _chk(a, torch.float32, "a"), _chk(w, torch.bfloat16, "w"), _chk(out, torch.float32, "out")
     if a_rows is not None:
         _chk(a_rows, torch.int32, "a_rows")
@@ -44,9 +45,14 @@ def linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, m: Optional[i
         _chk(e, torch.float32, "e")
         if e.numel() < (M - 1) * lde + e_off + (batch - 1) * e_batch + N:
             raise _lib.I64HError("linear: gate operand smaller than the launch reads")
+    if bias is not None:
+        _chk(bias, torch.float32, "bias")
+        if bias.numel() < (batch - 1) * bias_batch + N:
+            raise _lib.I64HError("linear: bias smaller than the launch reads")
     d = _lib.Linear(A=ptr(a) + 4 * a_off, lda=lda, a_rows=ptr(a_rows), W=ptr(w), C=ptr(out) + 4 * c_off, ldc=ldc, M=M, N=N, K=K, batch=batch,
                     a_batch=a_batch, w_batch=w_batch, c_batch=c_batch, exact=int(exact), epilogue=epilogue,
-                    E=(ptr(e) + 4 * e_off) if e is not None else 0, lde=lde, e_batch=e_batch, softcap=float(softcap))
+                    E=(ptr(e) + 4 * e_off) if e is not None else 0, lde=lde, e_batch=e_batch, softcap=float(softcap),
+                    bias=ptr(bias), bias_batch=int(bias_batch), scale=float(scale))
     call_dense("i64h_linear_run", _ref(d), _stream())
     return out
 
@@ -131,6 +137,181 @@ def latent_attn(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
 
 def latent_attn_workspace_floats(n: int, heads: int, kv_rank: int, splits: int) -> int:
     return int(_lib.load_dense().i64h_latent_attn_workspace_floats(n, heads, kv_rank, splits))
+
+
+# ---- recurrent and hybrid layers ----------------------------------------------------------------------------------------------------
+def _rows_ok(name: str, n: int, *tensors) -> None:
+    for t in tensors:
+        if t.numel() < n:
+            raise _lib.I64HError(f"{name}: a per-row operand has {t.numel()} entries, the launch has {n} rows")
+
+
+def embed_bigram(ids: torch.Tensor, positions: torch.Tensor, slot_ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, *,
+                 bigram: Optional[torch.Tensor] = None, buckets: int = 0, mul_prev: int = 0, mul_cur: int = 0,
+                 prev_token: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """See i64h_embed_bigram.  out fp32 [copies, n, W] (or [n, W]); prev_token int64 [slots], read and updated."""
+    _chk(ids, torch.int64, "ids"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
+    _chk(table, torch.bfloat16, "table"), _chk(out, torch.float32, "out")
+    n = ids.numel()
+    V, W = table.shape
+    _rows_ok("embed_bigram", n, positions, slot_ids)
+    copies = out.numel() // max(1, n * W)
+    if out.numel() != copies * n * W:
+        raise _lib.I64HError("embed_bigram: out is not [copies, n, W]")
+    if bigram is not None:
+        _chk(bigram, torch.bfloat16, "bigram"), _chk(prev_token, torch.int64, "prev_token")
+        if tuple(bigram.shape) != (buckets + 1, W):
+            raise _lib.I64HError(f"embed_bigram: table {tuple(bigram.shape)} for {buckets} buckets of width {W}")
+    d = _lib.EmbedBigram(ids=ptr(ids), positions=ptr(positions), slot_ids=ptr(slot_ids), table=ptr(table), V=V, W=W, bigram=ptr(bigram),
+                         buckets=int(buckets), mul_prev=int(mul_prev), mul_cur=int(mul_cur), prev_token=ptr(prev_token), out=ptr(out),
+                         copies=max(1, copies), n=n)
+    call_dense("i64h_embed_bigram", _ref(d), _stream())
+    return out
+
+
+def streams_step(streams: torch.Tensor, *, y: Optional[torch.Tensor] = None, y2: Optional[torch.Tensor] = None, yn_w: Optional[torch.Tensor] = None,
+                 y2n_w: Optional[torch.Tensor] = None, y_eps: float = 0.0, mix: Optional[torch.Tensor] = None, out_w: Optional[torch.Tensor] = None,
+                 in_w: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None, eps: float = 0.0, h: Optional[torch.Tensor] = None,
+                 rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """See i64h_streams_step.  streams fp32 [S, n, W], updated in place when y is given; h fp32 [n, W] (or [rows, W])."""
+    _chk(streams, torch.float32, "streams")
+    S, n, W = streams.shape
+    for t, name in ((y, "y"), (y2, "y2"), (yn_w, "yn_w"), (y2n_w, "y2n_w"), (mix, "mix"), (out_w, "out_w"), (in_w, "in_w"), (norm_w, "norm_w"), (h, "h")):
+        if t is not None:
+            _chk(t, torch.float32, name)
+    for t, name in ((y, "y"), (y2, "y2")):
+        if t is not None and (t.shape[-1] != W or t.numel() < n * W):
+            raise _lib.I64HError(f"streams_step: {name} is not [n, W]")
+    if (mix is not None and mix.numel() != S * S) or (out_w is not None and out_w.numel() != S) or (in_w is not None and in_w.numel() != S):
+        raise _lib.I64HError("streams_step: stream weights do not fit the number of streams")
+    if (yn_w is not None and yn_w.numel() != W) or (y2n_w is not None and y2n_w.numel() != W):
+        raise _lib.I64HError("streams_step: result norm weights are not [W]")
+    m_rows = n
+    if rows is not None:
+        _chk(rows, torch.int32, "rows")
+        m_rows = rows.numel()
+    if h is not None and h.numel() < m_rows * W:
+        raise _lib.I64HError("streams_step: h smaller than the rows it receives")
+    d = _lib.Streams(streams=ptr(streams), S=S, n=n, W=W, y=ptr(y), ldy=W, y2=ptr(y2), ldy2=W, yn_w=ptr(yn_w), y2n_w=ptr(y2n_w), y_eps=float(y_eps),
+                     mix=ptr(mix), out_w=ptr(out_w), in_w=ptr(in_w), norm_w=ptr(norm_w), norm_w_len=norm_w.numel() if norm_w is not None else 0,
+                     eps=float(eps), h=ptr(h), rows=ptr(rows), m_rows=m_rows)
+    call_dense("i64h_streams_step", _ref(d), _stream())
+    return h
+
+
+def causal_conv(p: torch.Tensor, *, off: int, channels: int, w: torch.Tensor, bias: Optional[torch.Tensor], positions: torch.Tensor,
+                slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: Optional[int] = None) -> torch.Tensor:
+    """See i64h_causal_conv.  p fp32 [n, ldp]; w fp32 [channels, taps]; state fp32 [slots, taps - 1, channels]; out fp32 [n, channels]."""
+    _chk(p, torch.float32, "p"), _chk(w, torch.float32, "w"), _chk(state, torch.float32, "state"), _chk(out, torch.float32, "out")
+    _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
+    rows = int(n if n is not None else positions.numel())
+    taps = w.shape[-1]
+    _rows_ok("causal_conv", rows, positions, slot_ids)
+    if bias is not None:
+        _chk(bias, torch.float32, "bias")
+    if w.shape[0] != channels or off + channels > p.shape[-1] or p.numel() < rows * p.shape[-1] or out.numel() < rows * channels or \
+            (bias is not None and bias.numel() != channels) or state.shape[-1] != channels or state.shape[-2] != max(taps - 1, 0):
+        raise _lib.I64HError("causal_conv: shapes do not fit the sizes")
+    d = _lib.CausalConv(P=ptr(p), ldp=p.shape[-1], off=off, channels=channels, taps=taps, w=ptr(w), bias=ptr(bias), positions=ptr(positions),
+                        slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=channels, n=rows)
+    call_dense("i64h_causal_conv", _ref(d), _stream())
+    return out
+
+
+def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, *, dt_off: int, lddt: int, dt_bias: torch.Tensor, a_log: torch.Tensor, d_skip: torch.Tensor,
+             heads: int, vdim: int, state: int, groups: int, seg_start: torch.Tensor, nseg: int, positions: torch.Tensor, slot_ids: torch.Tensor,
+             ssm_state: torch.Tensor, y: torch.Tensor, n: int) -> torch.Tensor:
+    """See i64h_ssm_scan.  xbc fp32 [n, heads * vdim + 2 * groups * state]; dt: the matrix whose columns [dt_off, + heads) hold the raw
+    steps (row stride lddt); ssm_state fp32 [slots, heads, state, vdim]; y fp32 [n, heads * vdim]."""
+    for t, name in ((xbc, "xbc"), (dt, "dt"), (dt_bias, "dt_bias"), (a_log, "a_log"), (d_skip, "d_skip"), (ssm_state, "ssm_state"), (y, "y")):
+        _chk(t, torch.float32, name)
+    _chk(seg_start, torch.int32, "seg_start"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
+    inner = heads * vdim
+    _rows_ok("ssm_scan", n, positions, slot_ids)
+    if xbc.shape[-1] != inner + 2 * groups * state or xbc.numel() < n * xbc.shape[-1] or y.numel() < n * inner or dt.numel() < (n - 1) * lddt + dt_off + heads or \
+            min(dt_bias.numel(), a_log.numel(), d_skip.numel()) < heads or tuple(ssm_state.shape[1:]) != (heads, state, vdim) or seg_start.numel() < nseg + 1:
+        raise _lib.I64HError("ssm_scan: shapes do not fit the sizes")
+    d = _lib.SsmScan(xbc=ptr(xbc), ldx=xbc.shape[-1], dt=ptr(dt) + 4 * dt_off, lddt=lddt, dt_bias=ptr(dt_bias), A_log=ptr(a_log), Dskip=ptr(d_skip),
+                     heads=heads, vdim=vdim, state=state, groups=groups, seg_start=ptr(seg_start), nseg=nseg, positions=ptr(positions),
+                     slot_ids=ptr(slot_ids), ssm_state=ptr(ssm_state), y=ptr(y), ldy=inner, n=n)
+    call_dense("i64h_ssm_scan", _ref(d), _stream())
+    return y
+
+
+def gate_norm(y: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, groups: int, eps: float, z: Optional[torch.Tensor] = None, z_off: int = 0,
+              ldz: int = 0, n: Optional[int] = None) -> torch.Tensor:
+    """out = rms_groups(y * silu(z)) * w: see i64h_gate_norm.  y, out fp32 [n, width]; z the columns [z_off, + width) of a matrix of row stride ldz."""
+    _chk(y, torch.float32, "y"), _chk(w, torch.float32, "w"), _chk(out, torch.float32, "out")
+    width = w.numel()
+    rows = int(n if n is not None else y.numel() // width)
+    if y.numel() < rows * width or out.numel() < rows * width:
+        raise _lib.I64HError("gate_norm: operand smaller than the launch reads or writes")
+    if z is not None:
+        _chk(z, torch.float32, "z")
+        if z.numel() < (rows - 1) * ldz + z_off + width:
+            raise _lib.I64HError("gate_norm: gate smaller than the launch reads")
+    d = _lib.GateNorm(y=ptr(y), ldy=width, z=(ptr(z) + 4 * z_off) if z is not None else 0, ldz=ldz, w=ptr(w), width=width, groups=groups, eps=float(eps),
+                      out=ptr(out), ldo=width, n=rows)
+    call_dense("i64h_gate_norm", _ref(d), _stream())
+    return out
+
+
+def mingru_scan(p: torch.Tensor, *, z_off: int, x_off: int, g_off: int, width: int, seg_start: torch.Tensor, nseg: int, positions: torch.Tensor,
+                slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor, n: int) -> torch.Tensor:
+    """See i64h_mingru_scan.  p fp32 [n, ldp]; state fp32 [slots, width]; out fp32 [n, width]."""
+    _chk(p, torch.float32, "p"), _chk(state, torch.float32, "state"), _chk(out, torch.float32, "out")
+    _chk(seg_start, torch.int32, "seg_start"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
+    _rows_ok("mingru_scan", n, positions, slot_ids)
+    if max(z_off, x_off, g_off) + width > p.shape[-1] or p.numel() < n * p.shape[-1] or out.numel() < n * width or state.shape[-1] != width or \
+            seg_start.numel() < nseg + 1:
+        raise _lib.I64HError("mingru_scan: shapes do not fit the sizes")
+    d = _lib.MinGruScan(P=ptr(p), ldp=p.shape[-1], z_off=z_off, x_off=x_off, g_off=g_off, width=width, seg_start=ptr(seg_start), nseg=nseg,
+                        positions=ptr(positions), slot_ids=ptr(slot_ids), state=ptr(state), out=ptr(out), ldo=width, n=n)
+    call_dense("i64h_mingru_scan", _ref(d), _stream())
+    return out
+
+
+def kattn_prep(p: torch.Tensor, *, q_off: int, k_off: int, heads: int, kv_heads: int, dim: int, q_norm_w: torch.Tensor, k_norm_w: torch.Tensor,
+               temp: Optional[torch.Tensor], scale: float, eps: float, positions: torch.Tensor, slot_ids: torch.Tensor, block_table: torch.Tensor,
+               cache: torch.Tensor, kscale: torch.Tensor, q: torch.Tensor, n: Optional[int] = None) -> None:
+    """See i64h_kattn_prep.  cache [blocks, block, kv_heads * dim] fp32 / bf16; kscale fp32 [blocks, block]; q fp32 [n, heads * dim]."""
+    _chk(p, torch.float32, "p"), _chk(q_norm_w, torch.float32, "q_norm_w"), _chk(k_norm_w, torch.float32, "k_norm_w"), _chk(q, torch.float32, "q")
+    _chk(kscale, torch.float32, "kscale"), _chk(cache, None, "cache")
+    _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids"), _chk(block_table, torch.int32, "block_table")
+    rows = int(n if n is not None else positions.numel())
+    _rows_ok("kattn_prep", rows, positions, slot_ids)
+    if temp is not None:
+        _chk(temp, torch.float32, "temp")
+    if cache.shape[-1] != kv_heads * dim or kscale.numel() != cache.shape[0] * cache.shape[1] or q.numel() < rows * heads * dim or \
+            q_norm_w.numel() != heads * dim or k_norm_w.numel() != kv_heads * dim or (temp is not None and temp.numel() != heads) or \
+            max(q_off + heads * dim, k_off + kv_heads * dim) > p.shape[-1] or p.numel() < rows * p.shape[-1]:
+        raise _lib.I64HError("kattn_prep: shapes do not fit the sizes")
+    d = _lib.KAttnPrep(P=ptr(p), ldp=p.shape[-1], q_off=q_off, k_off=k_off, heads=heads, kv_heads=kv_heads, dim=dim, q_norm_w=ptr(q_norm_w),
+                       k_norm_w=ptr(k_norm_w), temp=ptr(temp), scale=float(scale), eps=float(eps), positions=ptr(positions), slot_ids=ptr(slot_ids),
+                       block_table=ptr(block_table), max_blocks_per_seq=block_table.shape[1], block_size=cache.shape[-2], cache=ptr(cache),
+                       cache_dtype=CACHE_DTYPE_CODE[cache.dtype], kscale=ptr(kscale), Q=ptr(q), n=rows)
+    call_dense("i64h_kattn_prep", _ref(d), _stream())
+
+
+def kattn(q: torch.Tensor, cache: torch.Tensor, kscale: torch.Tensor, block_table: torch.Tensor, slot_ids: torch.Tensor, positions: torch.Tensor, *,
+          chunk: int, bias: Optional[torch.Tensor], sink: bool, heads: int, kv_heads: int, dim: int, out: torch.Tensor, n: Optional[int] = None) -> torch.Tensor:
+    """See i64h_kattn.  q, out fp32 [n, heads * dim]; bias fp32 [distances, heads]."""
+    _chk(q, torch.float32, "q"), _chk(out, torch.float32, "out"), _chk(cache, None, "cache"), _chk(kscale, torch.float32, "kscale")
+    _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids"), _chk(block_table, torch.int32, "block_table")
+    rows = int(n if n is not None else positions.numel())
+    _rows_ok("kattn", rows, positions, slot_ids)
+    if bias is not None:
+        _chk(bias, torch.float32, "bias")
+        if bias.dim() != 2 or bias.shape[1] != heads:
+            raise _lib.I64HError("kattn: bias is not [distances, heads]")
+    if cache.shape[-1] != kv_heads * dim or kscale.numel() != cache.shape[0] * cache.shape[1] or q.numel() < rows * heads * dim or out.numel() < rows * heads * dim:
+        raise _lib.I64HError("kattn: shapes do not fit the sizes")
+    d = _lib.KAttn(Q=ptr(q), cache=ptr(cache), cache_dtype=CACHE_DTYPE_CODE[cache.dtype], kscale=ptr(kscale), block_table=ptr(block_table),
+                   max_blocks_per_seq=block_table.shape[1], block_size=cache.shape[-2], slot_ids=ptr(slot_ids), positions=ptr(positions), chunk=int(chunk),
+                   bias=ptr(bias), bias_rows=bias.shape[0] if bias is not None else 0, sink=int(bool(sink)), out=ptr(out), n=rows, heads=heads,
+                   kv_heads=kv_heads, dim=dim)
+    call_dense("i64h_kattn", _ref(d), _stream())
+    return out
 
 
 def sample_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None, temperature: Optional[torch.Tensor] = None,

@@ -72,3 +72,24 @@ class LatentCache(PagePool):
         super().__init__(num_blocks, block, max_seqs, max(1, num_blocks), device)
         self.dtype, self.widths = dtype, [int(w) for w in widths]
         self.rows = [torch.zeros((num_blocks, block, w), dtype=dtype, device=device) for w in self.widths]
+
+
+class HybridCache(PagePool):
+    """Cache of a model whose layers keep different things: pages of key rows for attention layers (one row per token, which is also
+    the value, and the reciprocal root mean square of that row as a separate fp32 number), and per-slot state for recurrent layers
+    (fp32, one entry per sequence, overwritten by every step).  specs[l] = {"rows": width} and / or {"state": {name: shape}};
+    seq_state: per-slot state of the model as a whole, {name: (shape, dtype)}.  Recurrent state needs no clearing when a slot is used
+    again: the kernels take it as empty for a row at position 0."""
+
+    def __init__(self, specs: Sequence[dict], num_blocks: int, max_seqs: int, device, dtype=torch.bfloat16, block: int = 16, seq_state=None):
+        super().__init__(num_blocks, block, max_seqs, max(1, num_blocks), device)
+        self.dtype = dtype
+        self.rows: List = []
+        self.kscale: List = []
+        self.state: List[Dict[str, torch.Tensor]] = []
+        for sp in specs:
+            w = int(sp.get("rows", 0))
+            self.rows.append(torch.zeros((num_blocks, block, w), dtype=dtype, device=device) if w else None)
+            self.kscale.append(torch.zeros((num_blocks, block), dtype=torch.float32, device=device) if w else None)
+            self.state.append({k: torch.zeros((max_seqs, *shape), dtype=torch.float32, device=device) for k, shape in (sp.get("state") or {}).items()})
+        self.seq_state = {k: torch.zeros((max_seqs, *shape), dtype=dt, device=device) for k, (shape, dt) in (seq_state or {}).items()}

@@ -36,6 +36,14 @@ def _load_morilorn(config: dict, tensors, *, device, dtype, max_seqs, max_tokens
     return MorilornModel(cfg, tensors, device=device, dtype=dtype, max_seqs=max_seqs, num_kv_blocks=blocks, kv_block=kv_block)
 
 
+def _load_dogalorn(config: dict, tensors, *, device, dtype, max_seqs, max_tokens, kv_block=16, **_):
+    from .config import DogalornConfig
+    from .dogalorn import DogalornModel
+    cfg = DogalornConfig.from_dict(config)
+    blocks = max(1, (int(max_tokens) + kv_block - 1) // kv_block)
+    return DogalornModel(cfg, tensors, device=device, dtype=dtype, max_seqs=max_seqs, num_kv_blocks=blocks, kv_block=kv_block)
+
+
 def _load_complexity_deep(config: dict, tensors, *, device, dtype, max_seqs, max_tokens, quant="int8", **_):
     import torch
     from .checkpoint import config_from_dict, native_to_weights
@@ -47,6 +55,7 @@ def _load_complexity_deep(config: dict, tensors, *, device, dtype, max_seqs, max
 
 
 register("Morilorn", _load_morilorn)
+register("Dogalorn", _load_dogalorn)
 register("complexity-deep", _load_complexity_deep)
 register("ComplexityDeepModel", _load_complexity_deep)
 
