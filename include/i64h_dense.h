@@ -145,6 +145,14 @@ typedef struct {
     int32_t mode;
     int32_t splits;      /* mode 2: every token's keys are dealt to this many waves (tiles of 32 keys in turn) and merged by a second launch */
     float* workspace;    /* i64h_latent_attn_workspace_floats(n, heads, kv_rank, splits) floats when splits > 1 (NULL: no split) */
+    /* the same matrix-core kernel under key-valued attention (i64h_kattn below); all zero / NULL: latent attention as described */
+    int32_t row_stride;  /* values per cached row (0: kv_rank + rot_dim) */
+    int32_t kv_groups;   /* key heads side by side in a cached row, kv_rank + rot_dim values each; head h reads number h / (heads / kv_groups) */
+    int32_t chunk;       /* > 0: position p sees j <= p with j / chunk == p / chunk (the window is not used then) */
+    const float* kscale; /* per cached row: multiplies Q . row */
+    const float* bias;   /* fp32 [bias_rows, heads]: bias[min(p - j, bias_rows - 1), h] is added to the score */
+    int32_t bias_rows;
+    int32_t sink;        /* one more score of zero, without a value, in the softmax's denominator */
 } i64h_latent_attn_args;
 int i64h_set_latent_attn_decode_form(int32_t on); /* tuning / test knob: 1 (default) = mode 2 launches run the kernel that requests a tile's fragments a tile ahead; 0 = the general matrix-core kernel; same results up to summation order */
 int64_t i64h_latent_attn_workspace_floats(int64_t n, int32_t heads, int32_t kv_rank, int32_t splits);
@@ -318,7 +326,8 @@ int i64h_kattn_prep(const i64h_kattn_prep_args* d, void* stream);
 /* i64h_kattn: row t (position p) sees the cached positions j <= p of its sequence with j / chunk == p / chunk (chunk <= 0: all);
  *   s_j = Q[t, h] . k_j * kscale_j + bias[min(p - j, bias_rows - 1) * heads + h]      (bias fp32 [bias_rows, heads], may be NULL)
  *   w_j = exp(s_j) / (sink + sum_i exp(s_i))    (sink = 1: one more score of zero that carries no value; 0: the ordinary softmax)
- *   out[t, h, :] = sum_j w_j * k_j[g, :].   Scores, weights and sums fp32.  out fp32 [n, heads, dim]. */
+ *   out[t, h, :] = sum_j w_j * k_j[g, :].   Scores, weights and sums fp32.  out fp32 [n, heads, dim].
+ * The matrix-core form carries query and weights as two bf16 terms each (16 mantissa bits; products with the bf16 keys are exact). */
 typedef struct {
     const float* Q;
     const void* cache;
@@ -335,7 +344,13 @@ typedef struct {
     float* out;
     int64_t n;
     int32_t heads, kv_heads, dim;
+    int32_t mode;        /* 1: one wave per (row, head), fp32 products, any sizes and cache type; otherwise, where the cache is bf16 and dim % 16 == 0
+                            and <= 256, the matrix-core kernel of the latent attention: 3 a wave per 16 consecutive rows and head (portions of
+                            prompts), 0 / 2 a wave per token and 16 query heads of one key head (rows that are one per sequence) */
+    int32_t splits;      /* mode 0 / 2: every token's keys are dealt to this many waves and merged by a second launch */
+    float* workspace;    /* i64h_kattn_workspace_floats(n, heads, kv_heads, dim, splits) floats when splits > 1 */
 } i64h_kattn_args;
+int64_t i64h_kattn_workspace_floats(int64_t n, int32_t heads, int32_t kv_heads, int32_t dim, int32_t splits);
 int i64h_kattn(const i64h_kattn_args* d, void* stream);
 
 /* ---- sampling --------------------------------------------------------------------------------------------------------------

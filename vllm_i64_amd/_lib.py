@@ -251,7 +251,8 @@ class LatentAttn(ctypes.Structure):
     """Mirror of i64h_latent_attn_args (include/i64h_dense.h)."""
     _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("slot_ids", _P), ("positions", _P), ("window", _I), ("scale", _F), ("out", _P), ("n", _L), ("heads", _I), ("kv_rank", _I),
-                ("rot_dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P)]
+                ("rot_dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P), ("row_stride", _I), ("kv_groups", _I), ("chunk", _I), ("kscale", _P),
+                ("bias", _P), ("bias_rows", _I), ("sink", _I)]
 
 
 class EmbedBigram(ctypes.Structure):
@@ -302,14 +303,14 @@ class KAttn(ctypes.Structure):
     """Mirror of i64h_kattn_args (include/i64h_dense.h)."""
     _fields_ = [("Q", _P), ("cache", _P), ("cache_dtype", _I), ("kscale", _P), ("block_table", _P), ("max_blocks_per_seq", _I), ("block_size", _I),
                 ("slot_ids", _P), ("positions", _P), ("chunk", _I), ("bias", _P), ("bias_rows", _I), ("sink", _I), ("out", _P), ("n", _L), ("heads", _I),
-                ("kv_heads", _I), ("dim", _I)]
+                ("kv_heads", _I), ("dim", _I), ("mode", _I), ("splits", _I), ("workspace", _P)]
 
 
 _dense: Optional[ctypes.CDLL] = None
 
 
 def dense_exported_symbols():
-    return ["i64h_last_error", "i64h_version", "i64h_device_check", "i64h_latent_attn_workspace_floats", *DENSE_SIGNATURES.keys()]
+    return ["i64h_last_error", "i64h_version", "i64h_device_check", "i64h_latent_attn_workspace_floats", "i64h_kattn_workspace_floats", *DENSE_SIGNATURES.keys()]
 
 
 def load_dense() -> ctypes.CDLL:
@@ -326,6 +327,8 @@ def load_dense() -> ctypes.CDLL:
     lib.i64h_device_check.restype = _I
     lib.i64h_latent_attn_workspace_floats.restype = _L
     lib.i64h_latent_attn_workspace_floats.argtypes = [_L, _I, _I, _I]
+    lib.i64h_kattn_workspace_floats.restype = _L
+    lib.i64h_kattn_workspace_floats.argtypes = [_L, _I, _I, _I, _I]
     for name, sig in DENSE_SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = _I

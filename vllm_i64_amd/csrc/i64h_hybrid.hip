@@ -464,6 +464,11 @@ int i64h_kattn_prep(const i64h_kattn_prep_args* dp, void* stream) {
     return 0;
 }
 
+int64_t i64h_kattn_workspace_floats(int64_t n, int32_t heads, int32_t kv_heads, int32_t dim, int32_t splits) {
+    if (splits <= 1 || kv_heads <= 0) return 0;
+    return n * kv_heads * ((heads / kv_heads + 15) / 16) * (int64_t)(splits > 64 ? 64 : splits) * 16 * (dim + 2);
+}
+
 int i64h_kattn(const i64h_kattn_args* dp, void* stream) {
     I64H_CHECK_ARG(dp != nullptr, "kattn: no descriptor");
     const i64h_kattn_args& d = *dp;
@@ -474,6 +479,15 @@ int i64h_kattn(const i64h_kattn_args* dp, void* stream) {
     I64H_CHECK_ARG(!d.bias || d.bias_rows > 0, "kattn: an empty bias table");
     I64H_CHECK_ARG(d.block_size > 0 && d.max_blocks_per_seq > 0, "kattn: bad paging");
     if (d.n == 0) return 0;
+    if (d.mode != 1 && d.cache_dtype == 2 && d.dim % 16 == 0 && d.dim <= 256 && (uintptr_t)d.Q % 16 == 0 && (uintptr_t)d.cache % 16 == 0) {
+        i64h_latent_attn_args a = {};
+        a.Q = d.Q, a.cache = d.cache, a.cache_dtype = d.cache_dtype, a.block_table = d.block_table, a.max_blocks_per_seq = d.max_blocks_per_seq;
+        a.block_size = d.block_size, a.slot_ids = d.slot_ids, a.positions = d.positions, a.window = 0, a.scale = 1.0f, a.out = d.out, a.n = d.n;
+        a.heads = d.heads, a.kv_rank = d.dim, a.rot_dim = 0, a.mode = d.mode == 3 ? 3 : 2, a.splits = d.splits, a.workspace = d.workspace;
+        a.row_stride = d.kv_heads * d.dim, a.kv_groups = d.kv_heads, a.chunk = d.chunk, a.kscale = d.kscale, a.bias = d.bias, a.bias_rows = d.bias_rows;
+        a.sink = d.sink;
+        return i64h_latent_attn(&a, stream);
+    }
     const int64_t items = d.n * d.heads;
     const dim3 grid((unsigned)((items + 3) / 4));
     if (d.cache_dtype == 0) hipLaunchKernelGGL((kattn_row_kernel<float>), grid, dim3(256), 0, (hipStream_t)stream, d);

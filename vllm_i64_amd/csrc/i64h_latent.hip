@@ -182,16 +182,21 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     int* rowoff = info + 32;
     const int64_t task = blockIdx.x;
     const int split = blockIdx.y;
-    const int hgroups = (H + 15) / 16;
+    // key heads side by side in a cached row (key-valued attention): a head tile takes 16 of the rep query heads of ONE key head
+    const int G = p.kv_groups > 1 ? p.kv_groups : 1, rep = H / G, tpg = (rep + 15) / 16;
+    const int hgroups = G * tpg;
+    const int rstride = p.row_stride > 0 ? p.row_stride : D;
+    const int coff = (row_tiles ? (int)(task % H) / rep : (int)(task % hgroups) / tpg) * D;
+    const int hbase = row_tiles ? (int)(task % H) : ((int)(task % hgroups) / tpg) * rep + ((int)(task % hgroups) % tpg) * 16;
     auto row_of = [&](int m, int64_t& tok, int& head) -> bool {
         if (row_tiles) {     // the heads of a row tile are neighbours in the launch: they walk the same cached rows at the same time
             tok = (task / H) * 16 + m;
-            head = (int)(task % H);
+            head = hbase;
             return tok < p.n;
         }
         tok = task / hgroups;
-        head = (int)(task % hgroups) * 16 + m;
-        return head < H;
+        head = hbase + m;
+        return ((int)(task % hgroups) % tpg) * 16 + m < rep;
     };
     int64_t tok_n;
     int head_n;
@@ -226,12 +231,17 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
     for (int nb = 0; nb < LT_NB; ++nb) acc[nb] = lt_v4f{0, 0, 0, 0};
     float mrow[4], lrow[4];
+    int lor[4], hrow[4];   // per row of the tile: the first position it sees, its head (for the bias table)
+    const bool sink = p.sink && split == 0;     // the extra score of zero counts once: in the first share of the keys
+    __syncthreads();
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-        mrow[g] = -INFINITY;
-        lrow[g] = 0.0f;
+        mrow[g] = sink ? 0.0f : -INFINITY;
+        lrow[g] = sink ? 1.0f : 0.0f;
+        const int pp = info[kg * 4 + g];
+        lor[g] = p.chunk > 0 ? (max(pp, 0) / p.chunk) * p.chunk : (win > 0 ? max(0, pp - win + 1) : 0);
+        hrow[g] = min(row_tiles ? hbase : hbase + kg * 4 + g, H - 1);
     }
-    __syncthreads();
     const uint16_t* cache = (const uint16_t*)p.cache;
     int s0 = 0;
     while (s0 < 16) {
@@ -246,7 +256,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         for (int i = s0; i < s1; ++i) {
             const int pp = info[i];
             hi = max(hi, pp);
-            lo = min(lo, win > 0 ? max(0, pp - win + 1) : 0);
+            lo = min(lo, p.chunk > 0 ? (pp / p.chunk) * p.chunk : (win > 0 ? max(0, pp - win + 1) : 0));
         }
         const int32_t* bt = p.block_table + (int64_t)sl * p.max_blocks_per_seq;
         for (int kb = (lo & ~31) + 32 * split; kb <= hi; kb += 32 * splits) {
@@ -256,10 +266,15 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             }
             __syncthreads();
             lt_v4f S[2];
+            float ksc[2] = {1.0f, 1.0f};
+            if (p.kscale) {
+                ksc[0] = p.kscale[rowoff[n]];
+                ksc[1] = p.kscale[rowoff[16 + n]];
+            }
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 S[b] = lt_v4f{0, 0, 0, 0};
-                const uint16_t* rowp = cache + (int64_t)rowoff[16 * b + n] * D;
+                const uint16_t* rowp = cache + (int64_t)rowoff[16 * b + n] * rstride + coff;
 #pragma unroll
                 for (int ks = 0; ks < LT_KD; ++ks) {
                     if (ks * 32 < D) {
@@ -285,8 +300,10 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 #pragma unroll
                 for (int b = 0; b < 2; ++b) {
                     const int j = kb + 16 * b + n;
-                    const bool vis = in_run && j <= pr && (win <= 0 || pr - j < win);
-                    sv[b] = vis ? S[b][g] : -INFINITY;
+                    const bool vis = in_run && j <= pr && j >= lor[g];
+                    float sc = S[b][g] * ksc[b];
+                    if (p.bias) sc += 1.4426950408889634f * p.bias[(int64_t)min(max(pr - j, 0), p.bias_rows - 1) * H + hrow[g]];
+                    sv[b] = vis ? sc : -INFINITY;
                 }
                 const float mx = row16_max(fmaxf(sv[0], sv[1]));
                 const float mn = fmaxf(mrow[g], mx);
@@ -525,11 +542,13 @@ __global__ __launch_bounds__(64) void latent_attn_merge_kernel(const i64h_latent
     __shared__ float sf[64];
     const int lane = threadIdx.x;
     const int r = p.kv_rank, H = p.heads;
-    const int hgroups = (H + 15) / 16;
+    const int G = p.kv_groups > 1 ? p.kv_groups : 1, rep = H / G, tpg = (rep + 15) / 16;
+    const int hgroups = G * tpg;
     const int64_t task = blockIdx.x, tok = task / hgroups;
     const int m = blockIdx.y;
-    const int head = (int)(task % hgroups) * 16 + m;
-    if (head >= H) return;
+    const int sub = (int)(task % hgroups);
+    if ((sub % tpg) * 16 + m >= rep) return;
+    const int head = (sub / tpg) * rep + (sub % tpg) * 16 + m;
     const float* w = p.workspace + (task * splits * 16 + m) * (r + 2);      // share s: + s * 16 * (r + 2)
     const int64_t stride = (int64_t)16 * (r + 2);
     const float* mine = w + (int64_t)min(lane, splits - 1) * stride;
@@ -588,14 +607,19 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
     if (d.n == 0) return 0;
     const int D = d.kv_rank + d.rot_dim;
     const bool mfma_ok = d.cache_dtype == 2 && D % 8 == 0 && d.kv_rank % 16 == 0 && d.kv_rank <= 16 * LT_NB && D <= 32 * LT_KD &&
-                         (uintptr_t)d.Q % 16 == 0 && (uintptr_t)d.cache % 16 == 0;
+                         (uintptr_t)d.Q % 16 == 0 && (uintptr_t)d.cache % 16 == 0 && d.row_stride % 8 == 0;
+    I64H_CHECK_ARG(mfma_ok || d.mode == 1 || (d.kv_groups <= 1 && d.row_stride <= 0 && d.chunk <= 0 && !d.kscale && !d.bias && !d.sink),
+                   "latent_attn: key heads, chunks, key scales, bias and sink are built for the matrix-core form only");
     if (d.mode != 1 && mfma_ok) {
         const int row_tiles = d.mode == 3;
-        const int64_t tasks = row_tiles ? (d.n + 15) / 16 * d.heads : d.n * ((d.heads + 15) / 16);
+        const int G = d.kv_groups > 1 ? d.kv_groups : 1;
+        I64H_CHECK_ARG(d.heads % G == 0, "latent_attn: %d heads over %d key heads", d.heads, G);
+        const int64_t tasks = row_tiles ? (d.n + 15) / 16 * d.heads : d.n * G * ((d.heads / G + 15) / 16);
         I64H_CHECK_ARG(tasks < (1ll << 31), "latent_attn: too many tiles");
         const int splits = (!row_tiles && d.workspace && d.splits > 1) ? (d.splits > 64 ? 64 : d.splits) : 1;
         const size_t bytes = (size_t)d.kv_rank * LT_VLD * 2 + 2 * 16 * LT_VLD * 2 + 64 * 4;
-        if (row_tiles || !g_decode_form)
+        const bool plain = G == 1 && d.row_stride <= 0 && d.chunk <= 0 && !d.kscale && !d.bias && !d.sink;   // what the prefetching kernel covers
+        if (row_tiles || !g_decode_form || !plain)
             hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, row_tiles, splits);
         else
             hipLaunchKernelGGL(latent_attn_mfma_decode_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, splits);

@@ -28,6 +28,7 @@ import torch
 
 from . import ops_dense as D
 from .config import DogalornConfig
+from .model import attention_segments
 from .paged_cache import HybridCache
 
 
@@ -38,13 +39,15 @@ def distance_bias_table(rel: torch.Tensor, far: float) -> torch.Tensor:
     R = rel.shape[0]
     half = R // 2
     top = max(int(math.ceil(far)), half) + 1
-    n = torch.arange(top, dtype=torch.float32)
-    if half > 0 and far > half:
-        up = half + torch.floor(torch.log(torch.clamp(n, min=1.0) / half) / math.log(far / half) * (R - half)).to(torch.int64)
-    else:
-        up = torch.full((top,), R - 1, dtype=torch.int64)
-    bucket = torch.where(n < half, n.to(torch.int64), torch.clamp(up, max=R - 1))
-    return rel.to(torch.float32)[bucket].contiguous()
+    bucket = []
+    for n in range(top):
+        if n < half:
+            bucket.append(n)
+        elif half > 0 and far > half:
+            bucket.append(min(R - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (R - half)))))
+        else:
+            bucket.append(R - 1)
+    return rel.to(torch.float32)[torch.tensor(bucket, dtype=torch.int64)].contiguous()
 
 
 class _StepBuffers:
@@ -62,10 +65,13 @@ class _StepBuffers:
         self.act = torch.empty(n * max(model.max_ff, 1), **f32)
         self.xf = torch.empty(m, W, **f32)
         self.logits = torch.empty(m, model.cfg.vocab, **f32)
+        self.attn_ws: Dict[tuple, torch.Tensor] = {}   # partial results of split attention launches by (rows, heads, key heads, dim, splits)
 
 
 class DogalornModel:
     MAX_BUFFER_SETS = int(os.environ.get("I64H_MAX_BUFFER_SETS", "8"))
+    ATTN_MAX_SEGMENTS = 4     # more runs than this in one step (finely interleaved kinds) collapse into one launch
+    ATTN_WAVES = 1024         # waves a decode-sized attention launch aims at (256 CUs, four SIMDs each)
 
     def __init__(self, cfg: DogalornConfig, weights: Dict[str, torch.Tensor], device="cuda:0", dtype: str = "bfloat16", max_seqs: int = 4,
                  num_kv_blocks: int = 256, kv_block: int = 16, cache_dtype: Optional[torch.dtype] = None):
@@ -89,15 +95,11 @@ class DogalornModel:
         self.embed, self.head = bf(need("embed", (cfg.vocab, W))), bf(need("head", (cfg.vocab, W)))
         self.final_norm = f(need("final.norm", ()).reshape(1))
         self.bigram = bf(need("bigram", (cfg.bigram.buckets + 1, W))) if cfg.bigram is not None else None
-        own: Dict[int, dict] = {}
+        own = {i: self._load_layer(i, L, weights, need, bf, f) for i, L in enumerate(cfg.layers) if L.weights_of is None}
         self.layers: List[dict] = []
         specs = []
         for i, L in enumerate(cfg.layers):
-            if L.weights_of is not None:
-                d = own[L.weights_of]
-            else:
-                d = own[i] = self._load_layer(i, L, weights, need, bf, f)
-            self.layers.append(d)
+            self.layers.append(own[i if L.weights_of is None else L.weights_of])     # a borrowed layer: the same tensors, its own cache and state
             if L.type == "mamba2":
                 m = L.mixer
                 specs.append({"state": {"conv": (max(m.conv - 1, 0), m.conv_channels), "ssm": (m.heads, m.state, m.vdim)}})
@@ -177,6 +179,13 @@ class DogalornModel:
     def check_sync(self, force: bool = True):
         """No launch of this runner waits on a grid barrier: nothing to read back."""
 
+    def snapshot_state(self):
+        """The per-sequence recurrent state, for a caller that runs a step which must not count (a warm-up before a graph capture)."""
+        return self.kv.snapshot()
+
+    def restore_state(self, held) -> None:
+        self.kv.restore(held)
+
     def _runs(self, n: int, slot_ids: torch.Tensor, tokens_per_seq, rows_are_slots: bool):
         """First rows of the runs of consecutive rows of one sequence, int32 [runs + 1] on the device, and their number."""
         if rows_are_slots:
@@ -216,7 +225,7 @@ class DogalornModel:
         D.gate_norm(y, d["norm"], g, groups=m.norm_groups, eps=self.cfg.norm_eps, z=P, z_off=0, ldz=m.in_width, n=n)
         D.linear(g, d["o"], B.y, exact=ex)
 
-    def _parallel(self, B, d, l, n, positions, slot_ids, kvc, seg, nseg) -> None:
+    def _parallel(self, B, d, l, n, positions, slot_ids, kvc, seg, nseg, runs, ctx_hint) -> None:
         a, g, ex = d["m"].left, d["m"].right, self.exact
         N1 = d["n_in"]
         P = B.p[: n * N1].view(n, N1)
@@ -227,8 +236,22 @@ class DogalornModel:
                      temp=d["temp"], scale=a.scale, eps=self.cfg.norm_eps, positions=positions, slot_ids=slot_ids, block_table=kvc.block_table,
                      cache=kvc.rows[l], kscale=kvc.kscale[l], q=Q, n=n)
         O = B.b[: n * nq].view(n, nq)
-        D.kattn(Q, kvc.rows[l], kvc.kscale[l], kvc.block_table, slot_ids, positions, chunk=a.chunk, bias=d["bias"], sink=True, heads=a.heads,
-                kv_heads=a.kv_heads, dim=a.dim, out=O, n=n)
+        # runs of rows that are one per sequence (a wave takes a token's query heads of one key head, the keys dealt to several waves) and
+        # runs of prompt portions (a wave takes 16 consecutive rows of one head), each one launch
+        for r0, r1, one_per_seq in runs:
+            splits, ws = 1, None
+            if one_per_seq and not ex:
+                keys = min(a.chunk, ctx_hint) if a.chunk > 0 else ctx_hint
+                tasks = (r1 - r0) * a.kv_heads * ((a.heads // a.kv_heads + 15) // 16)
+                splits = max(1, min(self.ATTN_WAVES // max(1, tasks), keys // 64, 64))
+                if splits > 1:
+                    key = (r1 - r0, a.heads, a.kv_heads, a.dim, splits)
+                    ws = B.attn_ws.get(key)
+                    if ws is None:
+                        ws = B.attn_ws[key] = torch.empty(max(1, D.kattn_workspace_floats(r1 - r0, a.heads, a.kv_heads, a.dim, splits)), dtype=torch.float32,
+                                                          device=self.device)
+            D.kattn(Q[r0:r1], kvc.rows[l], kvc.kscale[l], kvc.block_table, slot_ids[r0:r1], positions[r0:r1], chunk=a.chunk, bias=d["bias"], sink=True,
+                    heads=a.heads, kv_heads=a.kv_heads, dim=a.dim, out=O[r0:r1], n=r1 - r0, mode=2 if one_per_seq else 3, splits=splits, workspace=ws)
         D.linear(O, d["o_left"], B.y, exact=ex)
         R = B.c[: n * g.width].view(n, g.width)
         D.mingru_scan(P, z_off=d["z_off"], x_off=d["x_off"], g_off=d["g_off"], width=g.width, seg_start=seg, nseg=nseg, positions=positions,
@@ -254,6 +277,10 @@ class DogalornModel:
             return B.logits
         eps = cfg.norm_eps
         seg, nseg = self._runs(n, slot_ids, tokens_per_seq, rows_are_slots)
+        if tokens_per_seq is not None:
+            runs = attention_segments(tokens_per_seq, n, self.ATTN_MAX_SEGMENTS)
+        else:
+            runs = [(0, n, bool(rows_are_slots))]
         bg = cfg.bigram
         D.embed_bigram(token_ids, positions, slot_ids, self.embed, B.streams, bigram=self.bigram, buckets=bg.buckets if bg else 0,
                        mul_prev=bg.mul_prev if bg else 0, mul_cur=bg.mul_cur if bg else 0, prev_token=kvc.seq_state.get("prev_token"))
@@ -268,7 +295,7 @@ class DogalornModel:
                 if d["type"] == "mamba2":
                     self._mamba2(B, d, l, n, positions, slot_ids, kvc, seg, nseg)
                 else:
-                    self._parallel(B, d, l, n, positions, slot_ids, kvc, seg, nseg)
+                    self._parallel(B, d, l, n, positions, slot_ids, kvc, seg, nseg, runs, int(max_ctx_hint))
                     two = True
             else:
                 ff = d["mlp"].ff

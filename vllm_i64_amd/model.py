@@ -1199,6 +1199,8 @@ class GreedyDecoder:
             return
         # warm up eagerly on a side stream (allocates every buffer), restoring the state afterwards, then capture
         state = (self.tokens.clone(), self.positions.clone(), self.ctx_len.clone())
+        # a runner with recurrent layers advances per-sequence state in every step: the warm-up step must not count
+        held = self.m.snapshot_state() if hasattr(self.m, "snapshot_state") else None
         s = torch.cuda.Stream(device=self.m.device)
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
@@ -1206,6 +1208,8 @@ class GreedyDecoder:
         torch.cuda.current_stream().wait_stream(s)
         for dst, src in zip((self.tokens, self.positions, self.ctx_len), state):
             dst.copy_(src)
+        if held is not None:
+            self.m.restore_state(held)
         torch.cuda.synchronize()
         self.m.pin_buffers(self.batch, self.batch)   # the graph replays on these addresses
         self.graph = torch.cuda.CUDAGraph()

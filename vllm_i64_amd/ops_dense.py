@@ -294,7 +294,8 @@ def kattn_prep(p: torch.Tensor, *, q_off: int, k_off: int, heads: int, kv_heads:
 
 
 def kattn(q: torch.Tensor, cache: torch.Tensor, kscale: torch.Tensor, block_table: torch.Tensor, slot_ids: torch.Tensor, positions: torch.Tensor, *,
-          chunk: int, bias: Optional[torch.Tensor], sink: bool, heads: int, kv_heads: int, dim: int, out: torch.Tensor, n: Optional[int] = None) -> torch.Tensor:
+          chunk: int, bias: Optional[torch.Tensor], sink: bool, heads: int, kv_heads: int, dim: int, out: torch.Tensor, n: Optional[int] = None,
+          mode: int = 0, splits: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """See i64h_kattn.  q, out fp32 [n, heads * dim]; bias fp32 [distances, heads]."""
     _chk(q, torch.float32, "q"), _chk(out, torch.float32, "out"), _chk(cache, None, "cache"), _chk(kscale, torch.float32, "kscale")
     _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids"), _chk(block_table, torch.int32, "block_table")
@@ -306,12 +307,23 @@ def kattn(q: torch.Tensor, cache: torch.Tensor, kscale: torch.Tensor, block_tabl
             raise _lib.I64HError("kattn: bias is not [distances, heads]")
     if cache.shape[-1] != kv_heads * dim or kscale.numel() != cache.shape[0] * cache.shape[1] or q.numel() < rows * heads * dim or out.numel() < rows * heads * dim:
         raise _lib.I64HError("kattn: shapes do not fit the sizes")
+    if splits > 1:
+        need = kattn_workspace_floats(rows, heads, kv_heads, dim, splits)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.float32, device=q.device)
+        _chk(workspace, torch.float32, "workspace")
+        if workspace.numel() < need:
+            raise _lib.I64HError(f"kattn: workspace of {workspace.numel()} floats, {need} needed")
     d = _lib.KAttn(Q=ptr(q), cache=ptr(cache), cache_dtype=CACHE_DTYPE_CODE[cache.dtype], kscale=ptr(kscale), block_table=ptr(block_table),
                    max_blocks_per_seq=block_table.shape[1], block_size=cache.shape[-2], slot_ids=ptr(slot_ids), positions=ptr(positions), chunk=int(chunk),
                    bias=ptr(bias), bias_rows=bias.shape[0] if bias is not None else 0, sink=int(bool(sink)), out=ptr(out), n=rows, heads=heads,
-                   kv_heads=kv_heads, dim=dim)
+                   kv_heads=kv_heads, dim=dim, mode=int(mode), splits=int(splits) if splits > 1 else 1, workspace=ptr(workspace) if splits > 1 else 0)
     call_dense("i64h_kattn", _ref(d), _stream())
     return out
+
+
+def kattn_workspace_floats(n: int, heads: int, kv_heads: int, dim: int, splits: int) -> int:
+    return int(_lib.load_dense().i64h_kattn_workspace_floats(n, heads, kv_heads, dim, splits))
 
 
 def sample_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None, temperature: Optional[torch.Tensor] = None,

@@ -93,3 +93,14 @@ class HybridCache(PagePool):
             self.kscale.append(torch.zeros((num_blocks, block), dtype=torch.float32, device=device) if w else None)
             self.state.append({k: torch.zeros((max_seqs, *shape), dtype=torch.float32, device=device) for k, shape in (sp.get("state") or {}).items()})
         self.seq_state = {k: torch.zeros((max_seqs, *shape), dtype=dt, device=device) for k, (shape, dt) in (seq_state or {}).items()}
+
+    def _state_tensors(self) -> List[torch.Tensor]:
+        return [t for d in self.state for t in d.values()] + list(self.seq_state.values())
+
+    def snapshot(self) -> List[torch.Tensor]:
+        """Copies of every per-slot state tensor (not of the pages: writing a position's key again changes nothing)."""
+        return [t.clone() for t in self._state_tensors()]
+
+    def restore(self, held: List[torch.Tensor]) -> None:
+        for t, h in zip(self._state_tensors(), held):
+            t.copy_(h)
