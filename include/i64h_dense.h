@@ -239,7 +239,8 @@ int i64h_causal_conv(const i64h_causal_conv_args* d, void* stream);
  * Per sequence and head a (state x vdim) matrix S in fp32:  dt = softplus(dt_raw + dt_bias[a]),
  *   S <- exp(-exp(A_log[a]) * dt) * S + dt * B_t x_t^T,   y_t = S^T C_t + Dskip[a] * x_t,
  * x_t = xbc[t, a * vdim : +vdim], B_t = xbc[t, heads * vdim + g * state : +state], C_t = xbc[t, heads * vdim + (groups + g) * state : +state],
- * g = a / (heads / groups), dt_raw = dt[t, a].  ssm_state fp32 [slots, heads, state, vdim].  All arithmetic fp32. */
+ * g = a / (heads / groups), dt_raw = dt[t, a].  ssm_state fp32 [slots, heads, vdim, state] (S transposed; state <= 256).  All arithmetic fp32,
+ * the tokens of a sequence strictly in their order. */
 typedef struct {
     const float* xbc;
     int64_t ldx;

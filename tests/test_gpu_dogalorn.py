@@ -273,12 +273,12 @@ def _mamba_case(dev, heads, vdim, state, groups, conv, norm_groups, cut_sizes, s
          "dt_bias": torch.rand(heads, generator=g) * 3 - 2, "A_log": torch.rand(heads, generator=g) * 2.5 - 1.5, "D": torch.rand(heads, generator=g) + 0.5,
          "norm": torch.rand(inner, generator=g) + 0.5, "o": torch.eye(inner)}
     eps = 1e-5
-    lens = {3: 37, 1: 12}
+    lens = {3: 150, 1: 70}
     proj = {s: torch.randn(T, nin, generator=g) for s, T in lens.items()}
     want = {s: R.mamba2({k: v.double() for k, v in w.items()}, "", m, eps, proj[s].double()) for s in lens}
     cw, cb = w["conv"].to(dev), w["conv.b"].to(dev)
     conv_state = torch.full((4, max(conv - 1, 0), ch), 7.0, device=dev)       # stale contents: position 0 has to ignore them
-    ssm_state = torch.full((4, heads, state, vdim), -3.0, device=dev)
+    ssm_state = torch.full((4, heads, vdim, state), -3.0, device=dev)
     cuts = {s: cuts_of(T, cut_sizes) for s, T in lens.items()}
     got = {s: [] for s in lens}
     for k in range(max(len(c) for c in cuts.values())):
@@ -298,11 +298,13 @@ def _mamba_case(dev, heads, vdim, state, groups, conv, norm_groups, cut_sizes, s
         assert close(torch.cat(got[s]), want[s], 3e-5), (s, cut_sizes)
 
 
-@pytest.mark.parametrize("cut_sizes", [[64], [1], [2, 5, 1, 3], [7, 2]])
+@pytest.mark.parametrize("cut_sizes", [[64], [200], [1], [2, 5, 1, 3, 90], [7, 2]])
 def test_mamba2_mechanism_under_cuts(dev, cut_sizes):
     _mamba_case(dev, heads=6, vdim=10, state=6, groups=3, conv=3, norm_groups=2, cut_sizes=cut_sizes, seed=1)
     _mamba_case(dev, heads=2, vdim=64, state=16, groups=1, conv=5, norm_groups=1, cut_sizes=cut_sizes, seed=2)
     _mamba_case(dev, heads=1, vdim=3, state=130, groups=1, conv=1, norm_groups=3, cut_sizes=cut_sizes, seed=3)
+    _mamba_case(dev, heads=2, vdim=20, state=32, groups=2, conv=8, norm_groups=1, cut_sizes=cut_sizes, seed=4)
+    _mamba_case(dev, heads=1, vdim=17, state=7, groups=1, conv=11, norm_groups=1, cut_sizes=cut_sizes, seed=5)
 
 
 @pytest.mark.parametrize("cut_sizes", [[200], [1], [2, 9, 1, 30]])
@@ -312,7 +314,7 @@ def test_mingru_mechanism_under_cuts(dev, cut_sizes, width):
     g = torch.Generator().manual_seed(width)
     w = {"z": torch.eye(width), "x": torch.eye(width), "g": torch.eye(width), "o": torch.eye(width), "z.b": torch.zeros(width), "x.b": torch.zeros(width)}
     wd = {k: v.double() for k, v in w.items()}
-    lens = {0: 70, 2: 9}
+    lens = {0: 200, 2: 9}
     # the oracle projects one input three times; here the three projections are separate columns, so the oracle runs on a mechanism
     # of three equal projections and the product on three copies of the same columns
     h = {s: torch.randn(T, width, generator=g) * 2 for s, T in lens.items()}
@@ -522,7 +524,7 @@ def test_key_attention_sink_and_grouped_heads(dev):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_whole_prompt_and_layer_streams(dev, name, dtype):
     model = make_model(name, dtype, dev)
-    toks = tokens(name, 45, 1)
+    toks = tokens(name, 140, 1)
     layers = []
     want = oracle_logits(name, toks, layers=layers)
     model.kv.reserve(2, len(toks))

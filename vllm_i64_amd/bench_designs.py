@@ -1,6 +1,7 @@
-"""`bench.py --design morilorn`: prefill and decode throughput of the Morilorn design at layer sizes of real models (random weights),
-beside the package's closest existing model (the dense int8 decoder) at equal width, depth, feed-forward size and batch, and the
-design's kernels one by one against their rooflines beside the like kernel of that model.  Prints one JSON line."""
+"""`bench.py --design morilorn | dogalorn`: prefill and decode throughput of a registered design at layer sizes of real models (random
+weights), beside the package's closest existing model at equal width, depth, feed-forward size and batch (Morilorn: the dense int8
+decoder; Dogalorn: Morilorn, which shares its library, bf16 Linears and 32-bit residual), and the design's kernels one by one
+against their rooflines beside the like kernel of that model.  Prints one JSON line."""
 from __future__ import annotations
 
 import json
@@ -186,6 +187,156 @@ def run(args) -> dict:
     return result
 
 
+DOGALORN_SIZES = {
+    "w1024": dict(width=1024, blocks=4, ssm_heads=32, ssm_vdim=64, ssm_state=128, heads=16, kv_heads=4, dim=64, chunk=4096, gru_width=1024, ff=4096),
+    "w2048": dict(width=2048, blocks=2, ssm_heads=64, ssm_vdim=64, ssm_state=128, heads=32, kv_heads=8, dim=64, chunk=4096, gru_width=2048, ff=8192),
+}
+F32_TFLOPS = 157.0     # fp32 vector rate (what a recurrence that is not a matrix product can reach at most)
+
+
+def _dogalorn_kernels(sz, rows, batch, ctx, dev):
+    """Single launches at the step's shapes with the share of their roofline (matrix products: bf16 matrix peak; recurrences: the larger
+    of bytes / HBM rate and flop / fp32 vector rate; everything else: bytes / HBM rate), beside the like kernel of Morilorn."""
+    from . import ops_dense as D
+    W, ff, H, G, dm = sz["width"], sz["ff"], sz["heads"], sz["kv_heads"], sz["dim"]
+    Hs, P, N, R = sz["ssm_heads"], sz["ssm_vdim"], sz["ssm_state"], sz["gru_width"]
+    out = {}
+    g = torch.Generator(device=dev).manual_seed(1)
+    rn = lambda *s: torch.randn(*s, device=dev, generator=g)
+
+    def row(name, t, flops=0.0, bytes_=0.0, peak=BF16_TFLOPS):
+        share = max(flops / t / (peak * 1e12), bytes_ / t / (HBM_GBS * 1e9))
+        out[name] = {"us": round(t * 1e6, 1), "roofline_share": round(share, 3)}
+
+    seq = 512
+    warm_a, warm_w, warm_c = rn(rows, W), (rn(W, W) * 0.02).to(torch.bfloat16), torch.empty(rows, W, device=dev)
+    _time(lambda: D.linear(warm_a, warm_w, warm_c), 20)      # clocks and caches settle before the first timed launch
+    for n, tag in ((rows, "prefill"), (batch, "decode")):
+        nseq = n // seq if tag == "prefill" else n
+        per = seq if tag == "prefill" else 1
+        pos0 = 0 if tag == "prefill" else ctx - 1
+        pos = (torch.arange(per, dtype=torch.int32) + pos0).repeat(nseq).to(dev)
+        slots = torch.arange(nseq, dtype=torch.int32).repeat_interleave(per).to(dev)
+        seg = (torch.arange(nseq + 1, dtype=torch.int32) * per).to(dev)
+        reps = 5 if tag == "prefill" else 20
+        # feed-forward up-projection with bias and activation, beside Morilorn's gate / up pair
+        a = rn(n, W)
+        w_up, b_up = (rn(ff, W) * 0.02).to(torch.bfloat16), rn(ff)
+        act = torch.empty(n, ff, device=dev)
+        t = _time(lambda: D.linear(a, w_up, act, bias=b_up, epilogue=D.EPI_GELU_ERF), reps)
+        row(f"linear_up_bias_gelu_{tag}", t, flops=2.0 * n * ff * W, bytes_=2.0 * ff * W + 4.0 * n * (W + ff))
+        w_gu = (rn(2 * ff, W) * 0.02).to(torch.bfloat16)
+        t = _time(lambda: D.linear(a, w_gu, act, epilogue=D.EPI_GELU_MUL), reps)
+        row(f"morilorn_linear_gate_up_{tag}", t, flops=2.0 * n * 2 * ff * W, bytes_=2.0 * 2 * ff * W + 4.0 * n * (W + ff))
+        # multi-stream residual + norm, beside the gated post-norm
+        S = 2
+        st, y, h = rn(S, n, W), rn(n, W), torch.empty(n, W, device=dev)
+        mix, ow, iw, nw = torch.eye(S, device=dev), torch.ones(S, device=dev), torch.full((S,), 0.5, device=dev), torch.ones(1, device=dev)
+        t = _time(lambda: D.streams_step(st, y=y, mix=mix, out_w=ow, in_w=iw, norm_w=nw, eps=1e-6, h=h), reps)
+        row(f"streams_step_{tag}", t, bytes_=4.0 * n * W * (2 * S + 2))
+        gp, bb, nw2, o = rn(n, W), rn(W), rn(W), torch.empty(n, W, device=dev)
+        t = _time(lambda: D.gated_postnorm(st[0], nw2, 2, 1e-6, alpha=1.0, y=y, gate_pre=gp, ldg=W, gate_bias=bb, out=o), reps)
+        row(f"morilorn_gated_postnorm_{tag}", t, bytes_=4.0 * n * W * 4)
+        # state-space layer: convolution, recurrence, gate + norm
+        inner, ch = Hs * P, Hs * P + 2 * N
+        nin = inner + ch + Hs
+        Pm = rn(n, nin) * 0.5
+        cw, cb = rn(ch, 4) * 0.3, rn(ch) * 0.1
+        cstate, sstate = torch.zeros(nseq, 3, ch, device=dev), torch.zeros(nseq, Hs, P, N, device=dev)
+        xbc, yv, gv = torch.empty(n, ch, device=dev), torch.empty(n, inner, device=dev), torch.empty(n, inner, device=dev)
+        t = _time(lambda: D.causal_conv(Pm, off=inner, channels=ch, w=cw, bias=cb, positions=pos, slot_ids=slots, state=cstate, out=xbc, n=n), reps)
+        row(f"causal_conv_{tag}", t, bytes_=4.0 * n * ch * 2)
+        dtb, al, dk = torch.full((Hs,), -2.0, device=dev), torch.zeros(Hs, device=dev), torch.ones(Hs, device=dev)
+        t = _time(lambda: D.ssm_scan(xbc, Pm, dt_off=inner + ch, lddt=nin, dt_bias=dtb, a_log=al, d_skip=dk, heads=Hs, vdim=P, state=N, groups=1, seg_start=seg,
+                                     nseg=nseq, positions=pos, slot_ids=slots, ssm_state=sstate, y=yv, n=n), reps)
+        row(f"ssm_scan_{tag}", t, flops=6.0 * n * Hs * N * P, bytes_=4.0 * n * (ch + inner) + 8.0 * nseq * Hs * N * P, peak=F32_TFLOPS)
+        t = _time(lambda: D.gate_norm(yv, torch.ones(inner, device=dev), gv, groups=1, eps=1e-6, z=Pm, z_off=0, ldz=nin, n=n), reps)
+        row(f"gate_norm_{tag}", t, bytes_=4.0 * n * inner * 3)
+        # gated recurrence
+        Pg = rn(n, 3 * R)
+        gstate, go = torch.zeros(nseq, R, device=dev), torch.empty(n, R, device=dev)
+        t = _time(lambda: D.mingru_scan(Pg, z_off=0, x_off=R, g_off=2 * R, width=R, seg_start=seg, nseg=nseq, positions=pos, slot_ids=slots, state=gstate, out=go, n=n), reps)
+        row(f"mingru_scan_{tag}", t, bytes_=4.0 * n * R * 4)
+        # attention: a prompt's rows, and one row per sequence at context ctx, beside the latent attention
+        plen = seq if tag == "prefill" else ctx
+        nb = (plen + 15) // 16
+        bt = torch.arange(nseq * nb, dtype=torch.int32, device=dev).view(nseq, nb).contiguous()
+        kc = (rn(nseq * nb, 16, G * dm) * 0.5).to(torch.bfloat16)
+        ks = torch.rand(nseq * nb, 16, device=dev, generator=g) + 0.5
+        q, oa = rn(n, H * dm) * 0.3, torch.empty(n, H * dm, device=dev)
+        bias = torch.zeros(sz["chunk"] + 1, H, device=dev)
+        keys = seq * (seq + 1) / 2 * nseq if tag == "prefill" else float(min(ctx, sz["chunk"])) * n
+        sp = 1 if tag == "prefill" else max(1, min(4096 // max(1, n * G * ((H // G + 15) // 16)), int(keys / n) // 64, 64))
+        t = _time(lambda: D.kattn(q, kc, ks, bt, slots, pos, chunk=sz["chunk"], bias=bias, sink=True, heads=H, kv_heads=G, dim=dm, out=oa, n=n,
+                                  mode=3 if tag == "prefill" else 2, splits=sp), reps)
+        row(f"kattn_{tag}", t, flops=4.0 * keys * H * dm, bytes_=(2.0 * keys * G * dm if tag == "decode" else 0.0) + 8.0 * n * H * dm)
+        r, rd = 256, 32
+        Dc = r + rd
+        lc = (rn(nseq * nb, 16, Dc) * 0.5).to(torch.bfloat16)
+        q2, ol = rn(n, H, Dc) * 0.3, torch.empty(n, H, r, device=dev)
+        lkeys = keys if tag == "prefill" else float(min(ctx, 1024)) * n
+        sp2 = 1 if tag == "prefill" else max(1, min(1024 // max(1, n * ((H + 15) // 16)), int(lkeys / n) // 64, 64))
+        wsp = torch.empty(max(1, D.latent_attn_workspace_floats(n, H, r, sp2)), device=dev) if sp2 > 1 else None
+        t = _time(lambda: D.latent_attn(q2, lc, bt, slots, pos, window=1024, scale=0.1, heads=H, kv_rank=r, rot_dim=rd, out=ol, mode=3 if tag == "prefill" else 2,
+                                        splits=sp2, workspace=wsp), reps)
+        row(f"morilorn_latent_attn_{tag}", t, flops=2.0 * lkeys * H * (Dc + r), bytes_=(2.0 * lkeys * Dc if tag == "decode" else 0.0) + 4.0 * n * H * (Dc + r))
+    return out
+
+
+def run_dogalorn(args) -> dict:
+    from . import _lib, synth
+    from .dogalorn import DogalornModel
+    from .model import GreedyDecoder
+    from .morilorn import MorilornModel
+    _lib.load(), _lib.load_dense()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    batch, ctx, rows = args.batch, args.prompt_len, 4096
+    result = {"metric": "prefill / decode tokens/s of the Dogalorn design beside Morilorn at equal sizes", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+              "warmup": args.warmup, "dtype": "bf16 matrix products, fp32 residual / norms / recurrences / attention math (both designs)", "data": "synthetic",
+              "config": {"batch": batch, "context": ctx, "prefill_step": f"{rows} rows = {rows // 512} prompts of 512 tokens"}, "sizes": {}}
+    for name in (args.design_sizes.split(",") if args.design_sizes else sorted(DOGALORN_SIZES)):
+        sz = DOGALORN_SIZES[name]
+        need_tokens = batch * (ctx + args.steps + args.warmup + 64)
+
+        def fill_hybrid(m):
+            g = torch.Generator(device=dev).manual_seed(5)
+            for t in m.kv.rows:
+                if t is not None:
+                    t.copy_((0.5 * torch.randn(t.shape, device=dev, generator=g)).to(t.dtype))
+            for t in m.kv.kscale:
+                if t is not None:
+                    t.fill_(2.0)
+            for d in m.kv.state:
+                for t in d.values():
+                    t.copy_(0.1 * torch.randn(t.shape, device=dev, generator=g))
+
+        def fill_latent(m):
+            g = torch.Generator(device=dev).manual_seed(5)
+            for t in m.kv.rows:
+                t.copy_((0.5 * torch.randn(t.shape, device=dev, generator=g)).to(t.dtype))
+
+        cfg = synth.dogalorn_config(**sz)
+        model = DogalornModel(cfg, synth.make_dogalorn_weights(cfg), device=dev, dtype="bfloat16", max_seqs=batch, num_kv_blocks=need_tokens // 16)
+        p, d, ms = _steps(model, GreedyDecoder, batch, ctx, rows, 512, args.steps, args.warmup, fill_hybrid, cfg.vocab, dev)
+        entry = {"dogalorn": {"prefill_tokens_per_s": round(p, 1), "decode_tokens_per_s": round(d, 1), "decode_ms_per_step": round(ms, 3), "layers": cfg.num_layers,
+                              "shape": sz}}
+        del model
+        torch.cuda.empty_cache()
+        mcfg = synth.morilorn_config(width=sz["width"], layers=4 * sz["blocks"], heads=sz["heads"], dim=32, rot_dim=32, vdim=64, kv_rank=256, ff=sz["ff"], window=1024)
+        mm = MorilornModel(mcfg, synth.make_morilorn_weights(mcfg), device=dev, dtype="bfloat16", max_seqs=batch, num_kv_blocks=need_tokens // 16)
+        p, d, ms = _steps(mm, GreedyDecoder, batch, ctx, rows, 512, args.steps, args.warmup, fill_latent, mcfg.vocab, dev)
+        entry["morilorn"] = {"prefill_tokens_per_s": round(p, 1), "decode_tokens_per_s": round(d, 1), "decode_ms_per_step": round(ms, 3), "layers": mcfg.num_layers}
+        del mm
+        torch.cuda.empty_cache()
+        entry["kernels"] = _dogalorn_kernels(sz, rows, batch, ctx, dev)
+        result["sizes"][name] = entry
+    first = result["sizes"][sorted(result["sizes"])[0]]["dogalorn"]
+    result["value"], result["ms_per_step"] = first["decode_tokens_per_s"], first["decode_ms_per_step"]
+    result["higher_is_better"], result["scaling"], result["vs_baseline"] = True, "weak", None
+    return result
+
+
 def main(args) -> int:
-    print(json.dumps(run(args)), flush=True)
+    print(json.dumps(run_dogalorn(args) if args.design == "dogalorn" else run(args)), flush=True)
     return 0

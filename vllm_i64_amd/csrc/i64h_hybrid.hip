@@ -2,9 +2,9 @@
 //   embed_bigram_kernel / prev_token_kernel : token embedding + hashed bigram embedding; the previous token is per-sequence state
 //   streams_kernel        : multi-stream residual write + the next sublayer's weighted read and RMS norm, one workgroup per row
 //   causal_conv_kernel / conv_carry_kernel : per-channel causal convolution + silu over rows and carried inputs; the carry update
-//   ssm_scan_kernel       : state-space recurrence with a scalar decay per head, the (state x vdim) matrix of a head in LDS
+//   ssm_scan_kernel       : state-space recurrence with a scalar decay per head, a head's matrix in registers (16 lanes per value column)
 //   gate_norm_kernel      : y * silu(z) -> RMS norm in groups
-//   mingru_scan_kernel    : element-wise gated recurrence
+//   mingru_scan_kernel    : element-wise gated recurrence, tiles of 64 tokens scanned by four waves and folded
 //   kattn_prep_kernel     : whole-row RMS norms of query and key, key-norm weights / scale / temperature folded into the query,
 //                           raw key row and its 1 / rms into the paged cache
 //   kattn_row_kernel      : attention over the cached keys (which are also the values) with distance bias, chunk mask and sink
@@ -149,6 +149,36 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const i64h_causal_conv
     p.out[t * p.ldo + c] = hy_silu(a);
 }
 
+// the same for 2 .. 8 taps: a thread walks CV_ROWS consecutive rows of its channel with the weights and the last TAPS - 1 inputs in
+// registers; only the first row of the walk and the first row of a run look back through memory
+#define CV_ROWS 16
+template <int TAPS>
+__global__ __launch_bounds__(256) void causal_conv_walk_kernel(const i64h_causal_conv_args p) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= p.channels) return;
+    const int64_t t0 = (int64_t)blockIdx.y * CV_ROWS, t1 = min(p.n, t0 + CV_ROWS);
+    float w[TAPS], win[TAPS - 1];     // win[d - 1]: the input d positions back
+#pragma unroll
+    for (int k = 0; k < TAPS; ++k) w[k] = p.w[(int64_t)c * TAPS + k];
+    const float bias = p.bias ? p.bias[c] : 0.0f;
+    for (int64_t t = t0; t < t1; ++t) {
+        if (t == t0 || !hy_continues(p.slot_ids, p.positions, t, 1)) {
+            const int before = conv_rows_before(p, t);
+#pragma unroll
+            for (int d = 1; d < TAPS; ++d) win[d - 1] = conv_input(p, t, d, before, c);
+        }
+        const float x = p.P[t * p.ldp + p.off + c];
+        float a = bias;
+#pragma unroll
+        for (int k = 0; k < TAPS - 1; ++k) a += w[k] * win[TAPS - 2 - k];
+        a += w[TAPS - 1] * x;
+        p.out[t * p.ldo + c] = hy_silu(a);
+#pragma unroll
+        for (int d = TAPS - 2; d > 0; --d) win[d] = win[d - 1];
+        win[0] = x;
+    }
+}
+
 #define HY_MAX_TAPS 16
 __global__ __launch_bounds__(256) void conv_carry_kernel(const i64h_causal_conv_args p) {
     const int64_t t = blockIdx.y;
@@ -162,59 +192,81 @@ __global__ __launch_bounds__(256) void conv_carry_kernel(const i64h_causal_conv_
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
-// one workgroup per (head, run of rows): thread (lane over the state index, value column); the head's matrix stays in LDS
-__global__ __launch_bounds__(256) void ssm_scan_kernel(const i64h_ssm_scan_args p) {
-    extern __shared__ float sm[];
+// One workgroup per (head, 16 value columns, run of rows); a wave takes four columns, the 16 lanes of a DPP row share a column and
+// hold KPT consecutive state indices each in registers.  Per token a lane loads its own slices of B and C (the next token's while this
+// one is computed), updates its states and the row sums the partial outputs with DPP moves: no LDS and no barrier, the tokens of a
+// run in their order (the same sums in the same order however a prompt is cut).  State layout [slot, head, value column, state index].
+template <int KPT>
+__global__ __launch_bounds__(256) void ssm_scan_kernel(const i64h_ssm_scan_args p, const int ctiles, const int vec) {
     const int N = p.state, P = p.vdim;
-    const int nl = 256 / P;                  // threads per value column
-    float* sS = sm;                          // [N, P]
-    float* sB = sS + (int64_t)N * P;         // [N]
-    float* sC = sB + N;                      // [N]
-    float* sX = sC + N;                      // [P]
-    float* sY = sX + P;                      // [nl, P]
-    const int tid = threadIdx.x;
-    const int a = blockIdx.x, seg = blockIdx.y;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int nlane = lane & 15, cl = lane >> 4;
+    const int a = blockIdx.x / ctiles, seg = blockIdx.y;
+    const int col = (blockIdx.x % ctiles) * 16 + w * 4 + cl;
+    const bool cok = col < P;
     const int g = a / (p.heads / p.groups);
     const int64_t r0 = p.seg_start[seg], r1 = p.seg_start[seg + 1];
     if (r1 <= r0) return;
-    const int slot = p.slot_ids[r0];
-    float* gS = p.ssm_state + ((int64_t)slot * p.heads + a) * N * P;
-    const bool fresh = p.positions[r0] == 0;
-    for (int i = tid; i < N * P; i += 256) sS[i] = fresh ? 0.0f : gS[i];
-    const int col = tid % P, nlane = tid / P;
-    const bool active = nlane < nl;
-    const float dtb = p.dt_bias[a], Aneg = -expf(p.A_log[a]), Dk = p.Dskip[a];
+    const int n0 = nlane * KPT;
     const int inner = p.heads * P;
-    __syncthreads();
-    for (int64_t t = r0; t < r1; ++t) {
+    float S[KPT], Bc[KPT], Cc[KPT], Bn[KPT], Cn[KPT];
+    float* gS = p.ssm_state + (((int64_t)p.slot_ids[r0] * p.heads + a) * P + (cok ? col : 0)) * N;
+    const bool fresh = p.positions[r0] == 0;
+#pragma unroll
+    for (int k = 0; k < KPT; ++k) S[k] = (!fresh && cok && n0 + k < N) ? gS[n0 + k] : 0.0f;
+    const float dtb = p.dt_bias[a], Aneg = -expf(p.A_log[a]), Dk = p.Dskip[a];
+    const int boff = inner + g * N + n0, coff = inner + (p.groups + g) * N + n0;
+    auto fetch = [&](int64_t t, float (&B)[KPT], float (&C)[KPT], float& x, float& dtr) {
         const float* row = p.xbc + t * p.ldx;
-        for (int i = tid; i < N; i += 256) {
-            sB[i] = row[inner + g * N + i];
-            sC[i] = row[inner + (p.groups + g) * N + i];
-        }
-        if (tid < P) sX[tid] = row[a * P + tid];
-        const float dt = hy_softplus(p.dt[t * p.lddt + a] + dtb);
-        const float decay = expf(Aneg * dt);
-        __syncthreads();
-        if (active) {
-            const float xv = dt * sX[col];
-            float part = 0.0f;
-            for (int n = nlane; n < N; n += nl) {
-                const float s = decay * sS[n * P + col] + sB[n] * xv;
-                sS[n * P + col] = s;
-                part += s * sC[n];
+        if (vec) {      // KPT % 4 == 0 and every slice starts at a multiple of four floats and lies inside the row
+#pragma unroll
+            for (int k = 0; k < KPT; k += 4) {
+                float4 b = make_float4(0, 0, 0, 0), c = b;
+                if (n0 + k < N) {
+                    b = *(const float4*)(row + boff + k);
+                    c = *(const float4*)(row + coff + k);
+                }
+                B[k] = b.x, B[k + 1] = b.y, B[k + 2] = b.z, B[k + 3] = b.w;
+                C[k] = c.x, C[k + 1] = c.y, C[k + 2] = c.z, C[k + 3] = c.w;
             }
-            sY[nlane * P + col] = part;
+        } else {
+#pragma unroll
+            for (int k = 0; k < KPT; ++k) {
+                const bool ok = n0 + k < N;
+                B[k] = ok ? row[boff + k] : 0.0f;
+                C[k] = ok ? row[coff + k] : 0.0f;
+            }
         }
-        __syncthreads();
-        if (tid < P) {
-            float y = 0.0f;
-            for (int i = 0; i < nl; ++i) y += sY[i * P + tid];
-            p.y[t * p.ldy + a * P + tid] = y + Dk * sX[tid];
+        x = cok ? row[a * P + col] : 0.0f;
+        dtr = p.dt[t * p.lddt + a];
+    };
+    float x, dtr, xn = 0.0f, dtn = 0.0f;
+    fetch(r0, Bc, Cc, x, dtr);
+    for (int64_t t = r0; t < r1; ++t) {
+        if (t + 1 < r1) fetch(t + 1, Bn, Cn, xn, dtn);
+        const float dt = hy_softplus(dtr + dtb);
+        const float decay = expf(Aneg * dt);
+        const float xv = dt * x;
+        float part = 0.0f;
+#pragma unroll
+        for (int k = 0; k < KPT; ++k) {
+            S[k] = decay * S[k] + Bc[k] * xv;
+            part += S[k] * Cc[k];
         }
-        __syncthreads();
+        part = group_sum(part, 16);
+        if (nlane == 0 && cok) p.y[t * p.ldy + a * P + col] = part + Dk * x;
+#pragma unroll
+        for (int k = 0; k < KPT; ++k) {
+            Bc[k] = Bn[k];
+            Cc[k] = Cn[k];
+        }
+        x = xn, dtr = dtn;
     }
-    for (int i = tid; i < N * P; i += 256) gS[i] = sS[i];
+    if (cok) {
+#pragma unroll
+        for (int k = 0; k < KPT; ++k)
+            if (n0 + k < N) gS[n0 + k] = S[k];
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -244,23 +296,60 @@ __global__ __launch_bounds__(256) void gate_norm_kernel(const i64h_gate_norm_arg
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
+// One workgroup per (64 channels, run of rows), tiles of 4 x GR_TL tokens: every wave scans GR_TL consecutive tokens of the tile from
+// an empty state, keeping per token the pair (A_t, B_t) of S_t = A_t * S_in + B_t, the waves' end pairs meet in LDS, every wave folds
+// the pairs before its own onto the tile's incoming state and finishes its tokens.  All loads of a tile are in flight together.
+#define GR_TL 16
 __global__ __launch_bounds__(256) void mingru_scan_kernel(const i64h_mingru_scan_args p) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
+    __shared__ float sA[2][4][64], sB[2][4][64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int c = blockIdx.x * 64 + lane;
+    const bool cok = c < p.width;
     const int seg = blockIdx.y;
-    if (c >= p.width) return;
     const int64_t r0 = p.seg_start[seg], r1 = p.seg_start[seg + 1];
     if (r1 <= r0) return;
-    float* st = p.state + (int64_t)p.slot_ids[r0] * p.width + c;
-    float S = p.positions[r0] == 0 ? 0.0f : *st;
-    for (int64_t t = r0; t < r1; ++t) {
-        const float* row = p.P + t * p.ldp;
-        const float z = hy_sigmoid(row[p.z_off + c]);
-        const float u = row[p.x_off + c];
-        const float cand = u >= 0.0f ? u + 0.5f : hy_sigmoid(u);
-        S = (1.0f - z) * S + z * cand;
-        p.out[t * p.ldo + c] = S * hy_silu(row[p.g_off + c]);
+    float* st = p.state + (int64_t)p.slot_ids[r0] * p.width + (cok ? c : 0);
+    float carry = (p.positions[r0] == 0 || !cok) ? 0.0f : *st;
+    int buf = 0;
+    for (int64_t t0 = r0; t0 < r1; t0 += 4 * GR_TL, buf ^= 1) {
+        const int64_t tb = t0 + w * GR_TL;
+        const int cnt = cok ? (int)max((int64_t)0, min((int64_t)GR_TL, r1 - tb)) : 0;
+        float z[GR_TL], u[GR_TL], G[GR_TL], A[GR_TL], Bv[GR_TL];
+#pragma unroll
+        for (int i = 0; i < GR_TL; ++i) {
+            z[i] = u[i] = G[i] = 0.0f;
+            if (i < cnt) {
+                const float* row = p.P + (tb + i) * p.ldp;
+                z[i] = row[p.z_off + c];
+                u[i] = row[p.x_off + c];
+                G[i] = row[p.g_off + c];
+            }
+        }
+        float a = 1.0f, b = 0.0f;
+#pragma unroll
+        for (int i = 0; i < GR_TL; ++i) {
+            const float zz = i < cnt ? hy_sigmoid(z[i]) : 0.0f;      // past the end: the identity step
+            const float cand = u[i] >= 0.0f ? u[i] + 0.5f : hy_sigmoid(u[i]);
+            a = (1.0f - zz) * a;
+            b = (1.0f - zz) * b + zz * cand;
+            A[i] = a;
+            Bv[i] = b;
+        }
+        sA[buf][w][lane] = a;
+        sB[buf][w][lane] = b;
+        __syncthreads();      // (the buffers alternate: the next tile's writes cannot overtake this tile's reads)
+        float sin = carry, mine = carry;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            if (v == w) mine = sin;
+            sin = sA[buf][v][lane] * sin + sB[buf][v][lane];
+        }
+        carry = sin;
+#pragma unroll
+        for (int i = 0; i < GR_TL; ++i)
+            if (i < cnt) p.out[(tb + i) * p.ldo + c] = (A[i] * mine + Bv[i]) * hy_silu(G[i]);
     }
-    *st = S;
+    if (w == 0 && cok) *st = carry;
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
@@ -402,7 +491,18 @@ int i64h_causal_conv(const i64h_causal_conv_args* dp, void* stream) {
     I64H_CHECK_ARG(d.n <= 65535, "causal_conv: %lld rows in one launch (at most 65535)", (long long)d.n);
     if (d.n == 0) return 0;
     const dim3 grid((unsigned)((d.channels + 255) / 256), (unsigned)d.n);
-    hipLaunchKernelGGL(causal_conv_kernel, grid, dim3(256), 0, (hipStream_t)stream, d);
+    const dim3 walk((unsigned)((d.channels + 255) / 256), (unsigned)((d.n + CV_ROWS - 1) / CV_ROWS));
+    hipStream_t s = (hipStream_t)stream;
+    switch (d.n >= 4 * CV_ROWS ? d.taps : 0) {      // few rows: a thread per row and channel fills the chip better
+        case 2: hipLaunchKernelGGL(causal_conv_walk_kernel<2>, walk, dim3(256), 0, s, d); break;
+        case 3: hipLaunchKernelGGL(causal_conv_walk_kernel<3>, walk, dim3(256), 0, s, d); break;
+        case 4: hipLaunchKernelGGL(causal_conv_walk_kernel<4>, walk, dim3(256), 0, s, d); break;
+        case 5: hipLaunchKernelGGL(causal_conv_walk_kernel<5>, walk, dim3(256), 0, s, d); break;
+        case 6: hipLaunchKernelGGL(causal_conv_walk_kernel<6>, walk, dim3(256), 0, s, d); break;
+        case 7: hipLaunchKernelGGL(causal_conv_walk_kernel<7>, walk, dim3(256), 0, s, d); break;
+        case 8: hipLaunchKernelGGL(causal_conv_walk_kernel<8>, walk, dim3(256), 0, s, d); break;
+        default: hipLaunchKernelGGL(causal_conv_kernel, grid, dim3(256), 0, s, d); break;
+    }
     I64H_CHECK_LAUNCH();
     if (d.taps > 1) {
         hipLaunchKernelGGL(conv_carry_kernel, grid, dim3(256), 0, (hipStream_t)stream, d);
@@ -414,15 +514,25 @@ int i64h_causal_conv(const i64h_causal_conv_args* dp, void* stream) {
 int i64h_ssm_scan(const i64h_ssm_scan_args* dp, void* stream) {
     I64H_CHECK_ARG(dp != nullptr, "ssm_scan: no descriptor");
     const i64h_ssm_scan_args& d = *dp;
-    I64H_CHECK_ARG(d.heads > 0 && d.vdim > 0 && d.vdim <= 256 && d.state > 0 && d.groups > 0 && d.heads % d.groups == 0,
-                   "ssm_scan: heads %d, groups %d, state %d, vdim %d (at most 256)", d.heads, d.groups, d.state, d.vdim);
+    I64H_CHECK_ARG(d.heads > 0 && d.vdim > 0 && d.state > 0 && d.groups > 0 && d.heads % d.groups == 0,
+                   "ssm_scan: heads %d, groups %d, state %d, vdim %d", d.heads, d.groups, d.state, d.vdim);
     I64H_CHECK_ARG(d.xbc && d.dt && d.dt_bias && d.A_log && d.Dskip && d.seg_start && d.positions && d.slot_ids && d.ssm_state && d.y, "ssm_scan: null operand");
-    const int nl = 256 / d.vdim;
-    const size_t lds = ((size_t)d.state * d.vdim + 2 * (size_t)d.state + d.vdim + (size_t)nl * d.vdim) * 4;
-    I64H_CHECK_ARG(lds <= 64 * 1024, "ssm_scan: a head's state of %d x %d values does not fit the kernel's LDS buffer", d.state, d.vdim);
+    I64H_CHECK_ARG(d.state <= 16 * 16, "ssm_scan: state %d above 256", d.state);
     I64H_CHECK_ARG(d.nseg <= 65535, "ssm_scan: %d runs in one launch", d.nseg);
     if (d.nseg <= 0 || d.n == 0) return 0;
-    hipLaunchKernelGGL(ssm_scan_kernel, dim3((unsigned)d.heads, (unsigned)d.nseg), dim3(256), lds, (hipStream_t)stream, d);
+    const int ctiles = (d.vdim + 15) / 16;
+    const int kpt = (d.state + 15) / 16;
+    const dim3 grid((unsigned)(d.heads * ctiles), (unsigned)d.nseg);
+    const int inner = d.heads * d.vdim;
+    auto launch = [&](auto kern, int K) {
+        const int vec = K % 4 == 0 && d.state % 4 == 0 && d.ldx % 4 == 0 && inner % 4 == 0 && (uintptr_t)d.xbc % 16 == 0;
+        hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, d, ctiles, vec);
+    };
+    if (kpt <= 1) launch(ssm_scan_kernel<1>, 1);
+    else if (kpt <= 2) launch(ssm_scan_kernel<2>, 2);
+    else if (kpt <= 4) launch(ssm_scan_kernel<4>, 4);
+    else if (kpt <= 8) launch(ssm_scan_kernel<8>, 8);
+    else launch(ssm_scan_kernel<16>, 16);
     I64H_CHECK_LAUNCH();
     return 0;
 }
@@ -446,7 +556,7 @@ int i64h_mingru_scan(const i64h_mingru_scan_args* dp, void* stream) {
     I64H_CHECK_ARG(d.width > 0 && d.P && d.seg_start && d.positions && d.slot_ids && d.state && d.out, "mingru_scan: bad arguments");
     I64H_CHECK_ARG(d.nseg <= 65535, "mingru_scan: %d runs in one launch", d.nseg);
     if (d.nseg <= 0 || d.n == 0) return 0;
-    hipLaunchKernelGGL(mingru_scan_kernel, dim3((unsigned)((d.width + 255) / 256), (unsigned)d.nseg), dim3(256), 0, (hipStream_t)stream, d);
+    hipLaunchKernelGGL(mingru_scan_kernel, dim3((unsigned)((d.width + 63) / 64), (unsigned)d.nseg), dim3(256), 0, (hipStream_t)stream, d);
     I64H_CHECK_LAUNCH();
     return 0;
 }

@@ -222,14 +222,14 @@ def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, *, dt_off: int, lddt: int, dt_
              heads: int, vdim: int, state: int, groups: int, seg_start: torch.Tensor, nseg: int, positions: torch.Tensor, slot_ids: torch.Tensor,
              ssm_state: torch.Tensor, y: torch.Tensor, n: int) -> torch.Tensor:
     """See i64h_ssm_scan.  xbc fp32 [n, heads * vdim + 2 * groups * state]; dt: the matrix whose columns [dt_off, + heads) hold the raw
-    steps (row stride lddt); ssm_state fp32 [slots, heads, state, vdim]; y fp32 [n, heads * vdim]."""
+    steps (row stride lddt); ssm_state fp32 [slots, heads, vdim, state]; y fp32 [n, heads * vdim]."""
     for t, name in ((xbc, "xbc"), (dt, "dt"), (dt_bias, "dt_bias"), (a_log, "a_log"), (d_skip, "d_skip"), (ssm_state, "ssm_state"), (y, "y")):
         _chk(t, torch.float32, name)
     _chk(seg_start, torch.int32, "seg_start"), _chk(positions, torch.int32, "positions"), _chk(slot_ids, torch.int32, "slot_ids")
     inner = heads * vdim
     _rows_ok("ssm_scan", n, positions, slot_ids)
     if xbc.shape[-1] != inner + 2 * groups * state or xbc.numel() < n * xbc.shape[-1] or y.numel() < n * inner or dt.numel() < (n - 1) * lddt + dt_off + heads or \
-            min(dt_bias.numel(), a_log.numel(), d_skip.numel()) < heads or tuple(ssm_state.shape[1:]) != (heads, state, vdim) or seg_start.numel() < nseg + 1:
+            min(dt_bias.numel(), a_log.numel(), d_skip.numel()) < heads or tuple(ssm_state.shape[1:]) != (heads, vdim, state) or seg_start.numel() < nseg + 1:
         raise _lib.I64HError("ssm_scan: shapes do not fit the sizes")
     d = _lib.SsmScan(xbc=ptr(xbc), ldx=xbc.shape[-1], dt=ptr(dt) + 4 * dt_off, lddt=lddt, dt_bias=ptr(dt_bias), A_log=ptr(a_log), Dskip=ptr(d_skip),
                      heads=heads, vdim=vdim, state=state, groups=groups, seg_start=ptr(seg_start), nseg=nseg, positions=ptr(positions),

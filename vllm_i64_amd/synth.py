@@ -109,3 +109,56 @@ def make_morilorn_weights(cfg, seed: int = 0, std: float = 0.02) -> Dict[str, to
             w.update({p + "mlp.gate": rn(L.mlp.ff, W), p + "mlp.up": rn(L.mlp.ff, W), p + "mlp.down": rn(W, L.mlp.ff), p + "rg2": rn(W, W),
                       p + "rg2.b": torch.zeros(W, dtype=torch.bfloat16), p + "norm2": one(W)})
     return w
+
+
+def dogalorn_config(width: int = 1024, blocks: int = 4, ssm_heads: int = 32, ssm_vdim: int = 64, ssm_state: int = 128, heads: int = 16, kv_heads: int = 4,
+                    dim: int = 64, chunk: int = 4096, gru_width: int = 1024, ff: int = 4096, streams: int = 2, vocab: int = 32000, rel_rows: int = 32):
+    """A Dogalorn configuration with layers of a real model's proportions: `blocks` times (two state-space layers, two layers of
+    chunked attention beside a gated recurrence), every layer with a feed-forward (random weights: make_dogalorn_weights)."""
+    from .config import DogalornConfig
+    mlp = {"kind": "dense", "ff": ff}
+    ssm = {"type": "mamba2", "mixer": {"heads": ssm_heads, "vdim": ssm_vdim, "state": ssm_state, "groups": 1, "conv": 4, "norm_groups": 1}, "mlp": mlp}
+    par = {"type": "parallel", "mlp": mlp, "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "bias_max": float(chunk),
+                                                              "mask": {"size": chunk}}, "right": {"width": gru_width}}}
+    cfg = DogalornConfig.from_dict({"architecture": "Dogalorn", "vocab": vocab, "width": width, "layers": [ssm, ssm, par, par] * blocks, "streams": streams,
+                                    "norm": {"eps": 1e-6}, "logit_scale": 1.0, "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}})
+    cfg.rel_rows = rel_rows
+    return cfg
+
+
+def make_dogalorn_weights(cfg, seed: int = 0, std: float = 0.02) -> Dict[str, torch.Tensor]:
+    """bf16 N(0, std) matrices, norm weights 1, biases 0, stream weights that start as the ordinary residual (read the mean, write
+    to every stream, no mixing), decays exp(-exp(A_log) dt) around 0.9, distance bias 0."""
+    g = torch.Generator().manual_seed(seed)
+    W, S = cfg.width, cfg.streams
+
+    def rn(*shape):
+        return torch.empty(*shape, dtype=torch.float32).normal_(0.0, std, generator=g).to(torch.bfloat16)
+
+    one = lambda *n: torch.ones(*n, dtype=torch.bfloat16)
+    zero = lambda *n: torch.zeros(*n, dtype=torch.bfloat16)
+    w = {"embed": rn(cfg.vocab, W), "head": rn(cfg.vocab, W), "final.norm": one(())}
+    if cfg.bigram is not None:
+        w["bigram"] = rn(cfg.bigram.buckets + 1, W)
+    for i, L in enumerate(cfg.layers):
+        if L.weights_of is not None:
+            continue
+        p, m = f"l{i}.", L.mixer
+        for q in (1, 2) if L.mlp is not None else (1,):
+            w[f"{p}norm{q}"] = one(())
+            if S:
+                w.update({f"{p}hc{q}.in": torch.full((S,), 1.0 / S, dtype=torch.bfloat16), f"{p}hc{q}.out": one(S), f"{p}hc{q}.mix": torch.eye(S, dtype=torch.bfloat16)})
+        if L.type == "mamba2":
+            w.update({p + "mix.in": rn(m.in_width, W), p + "mix.conv": rn(m.conv_channels, m.conv) * 10, p + "mix.conv.b": zero(m.conv_channels),
+                      p + "mix.dt_bias": torch.full((m.heads,), -2.0, dtype=torch.bfloat16), p + "mix.A_log": zero(m.heads), p + "mix.D": one(m.heads),
+                      p + "mix.norm": one(m.inner), p + "mix.o": rn(W, m.inner)})
+        else:
+            a, r = m.left, m.right.width
+            nq, nk = a.heads * a.dim, a.kv_heads * a.dim
+            w.update({p + "mix.left.q": rn(nq, W), p + "mix.left.k": rn(nk, W), p + "mix.left.q.norm": one(nq), p + "mix.left.k.norm": one(nk),
+                      p + "mix.left.rel": zero(getattr(cfg, "rel_rows", 32), a.heads), p + "mix.left.temp": one(a.heads), p + "mix.left.o": rn(W, nq),
+                      p + "mix.right.z": rn(r, W), p + "mix.right.z.b": zero(r), p + "mix.right.x": rn(r, W), p + "mix.right.x.b": zero(r),
+                      p + "mix.right.g": rn(r, W), p + "mix.right.o": rn(W, r), p + "mix.left.out": one(W), p + "mix.right.out": one(W)})
+        if L.mlp is not None:
+            w.update({p + "mlp.up": rn(L.mlp.ff, W), p + "mlp.up.b": zero(L.mlp.ff), p + "mlp.down": rn(W, L.mlp.ff), p + "mlp.down.b": zero(W)})
+    return w
