@@ -406,20 +406,27 @@ def test_key_attention_matrix_core_form(dev, H, G, d, chunk, block, cut_sizes):
     want = R.chunked_bias_attention({k: v.double() for k, v in w.items()}, "", m, eps, h.double())
     from vllm_i64_amd import ops_dense as D
     from vllm_i64_amd.dogalorn import distance_bias_table
-    pages = KeyPages(dev, T, G * d, block, torch.bfloat16)
     bias = distance_bias_table(w["rel"], 30.0).to(dev)
-    outs = []
-    for p, c in cuts_of(T, cut_sizes):
-        r = Rows(dev, [(1, p, c)])
-        P = torch.cat([h[p:p + c] @ w["q"].T, h[p:p + c]], 1).to(dev).contiguous()
-        Q, O = torch.empty(c, H * d, device=dev), torch.empty(c, H * d, device=dev)
-        D.kattn_prep(P, q_off=0, k_off=H * d, heads=H, kv_heads=G, dim=d, q_norm_w=w["q.norm"].to(dev), k_norm_w=w["k.norm"].to(dev), temp=w["temp"].to(dev),
-                     scale=0.4, eps=eps, positions=r.pos, slot_ids=r.slots, block_table=pages.bt, cache=pages.rows, kscale=pages.kscale, q=Q, n=c)
-        mode, splits = (2, 3) if c == 1 else (3, 1)
-        D.kattn(Q, pages.rows, pages.kscale, pages.bt, r.slots, r.pos, chunk=chunk, bias=bias, sink=True, heads=H, kv_heads=G, dim=d, out=O, n=c, mode=mode,
-                splits=splits)
-        outs.append(O.cpu())
-    assert close(torch.cat(outs), want, 1e-4)
+    # single rows: the kernel that requests its tiles ahead (1), and the general kernel with a token's heads per wave (0)
+    for single_row_form in ((1, 0) if 1 in cut_sizes else (1,)):
+        D.call_dense("i64h_set_latent_attn_decode_form", single_row_form)
+        try:
+            pages = KeyPages(dev, T, G * d, block, torch.bfloat16)
+            outs = []
+            for p, c in cuts_of(T, cut_sizes):
+                r = Rows(dev, [(1, p, c)])
+                P = torch.cat([h[p:p + c] @ w["q"].T, h[p:p + c]], 1).to(dev).contiguous()
+                Q, O = torch.empty(c, H * d, device=dev), torch.empty(c, H * d, device=dev)
+                D.kattn_prep(P, q_off=0, k_off=H * d, heads=H, kv_heads=G, dim=d, q_norm_w=w["q.norm"].to(dev), k_norm_w=w["k.norm"].to(dev),
+                             temp=w["temp"].to(dev), scale=0.4, eps=eps, positions=r.pos, slot_ids=r.slots, block_table=pages.bt, cache=pages.rows,
+                             kscale=pages.kscale, q=Q, n=c)
+                mode, splits = (2, 3) if c == 1 else (3, 1)
+                D.kattn(Q, pages.rows, pages.kscale, pages.bt, r.slots, r.pos, chunk=chunk, bias=bias, sink=True, heads=H, kv_heads=G, dim=d, out=O, n=c,
+                        mode=mode, splits=splits)
+                outs.append(O.cpu())
+        finally:
+            D.call_dense("i64h_set_latent_attn_decode_form", 1)
+        assert close(torch.cat(outs), want, 1e-4), single_row_form
 
 
 def test_key_attention_matrix_core_form_batches_of_unequal_rows(dev):

@@ -192,31 +192,54 @@ __global__ __launch_bounds__(256) void conv_carry_kernel(const i64h_causal_conv_
 }
 
 // ---------------------------------------------------------------------------------------------------------------------------
-// One workgroup per (head, 16 value columns, run of rows); a wave takes four columns, the 16 lanes of a DPP row share a column and
-// hold KPT consecutive state indices each in registers.  Per token a lane loads its own slices of B and C (the next token's while this
-// one is computed), updates its states and the row sums the partial outputs with DPP moves: no LDS and no barrier, the tokens of a
-// run in their order (the same sums in the same order however a prompt is cut).  State layout [slot, head, value column, state index].
-template <int KPT>
+// One workgroup per (head, 16 * CPT value columns, run of rows).  The 16 lanes of a DPP row share CPT neighbouring columns and hold KPT
+// consecutive state indices of each in registers; a wave has four such rows.  Per token a lane loads its own slices of B and C once
+// for its CPT columns (the next token's while this one is computed), updates its states with fused multiply-adds and the row sums the
+// partial outputs with DPP moves: no LDS and no barrier, the tokens of a run strictly in their order (the same sums in the same order
+// however a prompt is cut).  Step sizes and decays of 64 tokens are computed at once, a token per lane, and read back lane by lane.
+// State layout [slot, head, value column, state index].
+template <int KPT, int CPT>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(const i64h_ssm_scan_args p, const int ctiles, const int vec) {
     const int N = p.state, P = p.vdim;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int nlane = lane & 15, cl = lane >> 4;
     const int a = blockIdx.x / ctiles, seg = blockIdx.y;
-    const int col = (blockIdx.x % ctiles) * 16 + w * 4 + cl;
-    const bool cok = col < P;
+    const int cbase = (blockIdx.x % ctiles) * 16 * CPT + (w * 4 + cl) * CPT;
     const int g = a / (p.heads / p.groups);
     const int64_t r0 = p.seg_start[seg], r1 = p.seg_start[seg + 1];
     if (r1 <= r0) return;
     const int n0 = nlane * KPT;
     const int inner = p.heads * P;
-    float S[KPT], Bc[KPT], Cc[KPT], Bn[KPT], Cn[KPT];
-    float* gS = p.ssm_state + (((int64_t)p.slot_ids[r0] * p.heads + a) * P + (cok ? col : 0)) * N;
+    float S[CPT][KPT];
+    float* gS = p.ssm_state + ((int64_t)p.slot_ids[r0] * p.heads + a) * P * N + n0;      // + column * N
     const bool fresh = p.positions[r0] == 0;
 #pragma unroll
-    for (int k = 0; k < KPT; ++k) S[k] = (!fresh && cok && n0 + k < N) ? gS[n0 + k] : 0.0f;
+    for (int j = 0; j < CPT; ++j) {
+        const bool cok = cbase + j < P;
+        const float* src = gS + (int64_t)(cok ? cbase + j : 0) * N;
+#pragma unroll
+        for (int k = 0; k < KPT; ++k) S[j][k] = 0.0f;
+        if (!fresh && cok) {
+            if (vec) {
+#pragma unroll
+                for (int k = 0; k < KPT; k += 4)
+                    if (n0 + k < N) {
+                        const float4 v = *(const float4*)(src + k);
+                        S[j][k] = v.x, S[j][k + 1] = v.y, S[j][k + 2] = v.z, S[j][k + 3] = v.w;
+                    }
+            } else {
+#pragma unroll
+                for (int k = 0; k < KPT; ++k)
+                    if (n0 + k < N) S[j][k] = src[k];
+            }
+        }
+    }
     const float dtb = p.dt_bias[a], Aneg = -expf(p.A_log[a]), Dk = p.Dskip[a];
     const int boff = inner + g * N + n0, coff = inner + (p.groups + g) * N + n0;
-    auto fetch = [&](int64_t t, float (&B)[KPT], float (&C)[KPT], float& x, float& dtr) {
+    struct Tok {
+        float B[KPT], C[KPT], x[CPT];
+    };
+    auto fetch = [&](int64_t t, Tok& q) {
         const float* row = p.xbc + t * p.ldx;
         if (vec) {      // KPT % 4 == 0 and every slice starts at a multiple of four floats and lies inside the row
 #pragma unroll
@@ -226,46 +249,66 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const i64h_ssm_scan_args 
                     b = *(const float4*)(row + boff + k);
                     c = *(const float4*)(row + coff + k);
                 }
-                B[k] = b.x, B[k + 1] = b.y, B[k + 2] = b.z, B[k + 3] = b.w;
-                C[k] = c.x, C[k + 1] = c.y, C[k + 2] = c.z, C[k + 3] = c.w;
+                q.B[k] = b.x, q.B[k + 1] = b.y, q.B[k + 2] = b.z, q.B[k + 3] = b.w;
+                q.C[k] = c.x, q.C[k + 1] = c.y, q.C[k + 2] = c.z, q.C[k + 3] = c.w;
             }
         } else {
 #pragma unroll
             for (int k = 0; k < KPT; ++k) {
                 const bool ok = n0 + k < N;
-                B[k] = ok ? row[boff + k] : 0.0f;
-                C[k] = ok ? row[coff + k] : 0.0f;
+                q.B[k] = ok ? row[boff + k] : 0.0f;
+                q.C[k] = ok ? row[coff + k] : 0.0f;
             }
         }
-        x = cok ? row[a * P + col] : 0.0f;
-        dtr = p.dt[t * p.lddt + a];
+#pragma unroll
+        for (int j = 0; j < CPT; ++j) q.x[j] = cbase + j < P ? row[a * P + cbase + j] : 0.0f;
     };
-    float x, dtr, xn = 0.0f, dtn = 0.0f;
-    fetch(r0, Bc, Cc, x, dtr);
-    for (int64_t t = r0; t < r1; ++t) {
-        if (t + 1 < r1) fetch(t + 1, Bn, Cn, xn, dtn);
-        const float dt = hy_softplus(dtr + dtb);
-        const float decay = expf(Aneg * dt);
-        const float xv = dt * x;
-        float part = 0.0f;
+    auto step = [&](int64_t t, const Tok& q, float dt, float decay) {
 #pragma unroll
-        for (int k = 0; k < KPT; ++k) {
-            S[k] = decay * S[k] + Bc[k] * xv;
-            part += S[k] * Cc[k];
-        }
-        part = group_sum(part, 16);
-        if (nlane == 0 && cok) p.y[t * p.ldy + a * P + col] = part + Dk * x;
+        for (int j = 0; j < CPT; ++j) {
+            const float xv = dt * q.x[j];
+            float part = 0.0f;
 #pragma unroll
-        for (int k = 0; k < KPT; ++k) {
-            Bc[k] = Bn[k];
-            Cc[k] = Cn[k];
+            for (int k = 0; k < KPT; ++k) {
+                S[j][k] = fmaf(decay, S[j][k], q.B[k] * xv);
+                part = fmaf(S[j][k], q.C[k], part);
+            }
+            part = group_sum(part, 16);
+            if (nlane == 0 && cbase + j < P) p.y[t * p.ldy + a * P + cbase + j] = part + Dk * q.x[j];
         }
-        x = xn, dtr = dtn;
+    };
+    auto lane_value = [](float v, int i) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), i)); };
+    for (int64_t tb = r0; tb < r1; tb += 64) {
+        const int cnt = (int)min((int64_t)64, r1 - tb);
+        float dtv = 0.0f, dec = 1.0f;
+        if (lane < cnt) {
+            dtv = hy_softplus(p.dt[(tb + lane) * p.lddt + a] + dtb);
+            dec = expf(Aneg * dtv);
+        }
+        Tok q0, q1;
+        fetch(tb, q0);
+        for (int i = 0; i < cnt; i += 2) {
+            if (i + 1 < cnt) fetch(tb + i + 1, q1);
+            step(tb + i, q0, lane_value(dtv, i), lane_value(dec, i));
+            if (i + 1 < cnt) {
+                if (i + 2 < cnt) fetch(tb + i + 2, q0);
+                step(tb + i + 1, q1, lane_value(dtv, i + 1), lane_value(dec, i + 1));
+            }
+        }
     }
-    if (cok) {
 #pragma unroll
-        for (int k = 0; k < KPT; ++k)
-            if (n0 + k < N) gS[n0 + k] = S[k];
+    for (int j = 0; j < CPT; ++j) {
+        if (cbase + j >= P) continue;
+        float* dst = gS + (int64_t)(cbase + j) * N;
+        if (vec) {
+#pragma unroll
+            for (int k = 0; k < KPT; k += 4)
+                if (n0 + k < N) *(float4*)(dst + k) = make_float4(S[j][k], S[j][k + 1], S[j][k + 2], S[j][k + 3]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < KPT; ++k)
+                if (n0 + k < N) dst[k] = S[j][k];
+        }
     }
 }
 
@@ -520,19 +563,28 @@ int i64h_ssm_scan(const i64h_ssm_scan_args* dp, void* stream) {
     I64H_CHECK_ARG(d.state <= 16 * 16, "ssm_scan: state %d above 256", d.state);
     I64H_CHECK_ARG(d.nseg <= 65535, "ssm_scan: %d runs in one launch", d.nseg);
     if (d.nseg <= 0 || d.n == 0) return 0;
-    const int ctiles = (d.vdim + 15) / 16;
     const int kpt = (d.state + 15) / 16;
+    const int cpt = d.vdim > 16 ? 2 : 1;             // columns per lane: B and C are loaded once for both
+    const int ctiles = (d.vdim + 16 * cpt - 1) / (16 * cpt);
     const dim3 grid((unsigned)(d.heads * ctiles), (unsigned)d.nseg);
     const int inner = d.heads * d.vdim;
     auto launch = [&](auto kern, int K) {
-        const int vec = K % 4 == 0 && d.state % 4 == 0 && d.ldx % 4 == 0 && inner % 4 == 0 && (uintptr_t)d.xbc % 16 == 0;
+        const int vec = K % 4 == 0 && d.state % 4 == 0 && d.ldx % 4 == 0 && inner % 4 == 0 && (uintptr_t)d.xbc % 16 == 0 && (uintptr_t)d.ssm_state % 16 == 0;
         hipLaunchKernelGGL(kern, grid, dim3(256), 0, (hipStream_t)stream, d, ctiles, vec);
     };
-    if (kpt <= 1) launch(ssm_scan_kernel<1>, 1);
-    else if (kpt <= 2) launch(ssm_scan_kernel<2>, 2);
-    else if (kpt <= 4) launch(ssm_scan_kernel<4>, 4);
-    else if (kpt <= 8) launch(ssm_scan_kernel<8>, 8);
-    else launch(ssm_scan_kernel<16>, 16);
+    if (cpt == 2) {
+        if (kpt <= 1) launch(ssm_scan_kernel<1, 2>, 1);
+        else if (kpt <= 2) launch(ssm_scan_kernel<2, 2>, 2);
+        else if (kpt <= 4) launch(ssm_scan_kernel<4, 2>, 4);
+        else if (kpt <= 8) launch(ssm_scan_kernel<8, 2>, 8);
+        else launch(ssm_scan_kernel<16, 2>, 16);
+    } else {
+        if (kpt <= 1) launch(ssm_scan_kernel<1, 1>, 1);
+        else if (kpt <= 2) launch(ssm_scan_kernel<2, 1>, 2);
+        else if (kpt <= 4) launch(ssm_scan_kernel<4, 1>, 4);
+        else if (kpt <= 8) launch(ssm_scan_kernel<8, 1>, 8);
+        else launch(ssm_scan_kernel<16, 1>, 16);
+    }
     I64H_CHECK_LAUNCH();
     return 0;
 }

@@ -380,11 +380,16 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
     int* rowoff = (int*)(Pl + 16 * LT_VLD);   // [2][32] cache rows of two tiles' keys
     const int64_t task = blockIdx.x;
     const int split = blockIdx.y;
-    const int hgroups = (H + 15) / 16;
+    const int G = p.kv_groups > 1 ? p.kv_groups : 1, rep = H / G, tpg = (rep + 15) / 16;
+    const int hgroups = G * tpg;
     const int64_t tok = task / hgroups;
-    const int head0 = (int)(task % hgroups) * 16;
+    const int sub = (int)(task % hgroups);
+    const int hin = (sub % tpg) * 16;               // first of this wave's heads within its key head
+    const int head0 = (sub / tpg) * rep + hin;
+    const int rstride = p.row_stride > 0 ? p.row_stride : D;
+    const int coff = (sub / tpg) * D;
     const int pos = p.positions[tok], slot = p.slot_ids[tok];
-    const int lo = win > 0 ? max(0, pos - win + 1) : 0, hi = pos;
+    const int lo = p.chunk > 0 ? (pos / p.chunk) * p.chunk : (win > 0 ? max(0, pos - win + 1) : 0), hi = pos;
     const int32_t* bt = p.block_table + (int64_t)slot * p.max_blocks_per_seq;
     const uint16_t* cache = (const uint16_t*)p.cache;
     const int step = 32 * splits;
@@ -399,7 +404,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
     auto request = [&](int buf) {
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
-            const uint16_t* rowp = cache + (int64_t)rowoff[buf * 32 + 16 * b + n] * D;
+            const uint16_t* rowp = cache + (int64_t)rowoff[buf * 32 + 16 * b + n] * rstride + coff;
 #pragma unroll
             for (int ks = 0; ks < LT_KD; ++ks) {
                 const int d0 = ks * 32 + kg * 8;
@@ -416,7 +421,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
     // the query of row n (head head0 + n) times scale * log2(e), as two bf16 terms - converted while the first tile travels
     uint4 Qh[LT_KD], Ql[LT_KD];
     {
-        const bool valid_n = head0 + n < H;
+        const bool valid_n = hin + n < rep;
         const float* q = p.Q + (tok * H + head0 + n) * D;
         const float qs = p.scale * 1.4426950408889634f;
 #pragma unroll
@@ -440,15 +445,23 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
 #pragma unroll
     for (int nb = 0; nb < LT_NB; ++nb) acc[nb] = lt_v4f{0, 0, 0, 0};
     float mrow[4], lrow[4];
+    int hrow[4];
+    const bool sink = p.sink && split == 0;     // the extra score of zero counts once: in the first share of the keys
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-        mrow[g] = -INFINITY;
-        lrow[g] = 0.0f;
+        mrow[g] = sink ? 0.0f : -INFINITY;
+        lrow[g] = sink ? 1.0f : 0.0f;
+        hrow[g] = min(head0 + kg * 4 + g, H - 1);
     }
     int it = 0;
     for (int kb = kb0; kb <= hi; kb += step, ++it) {
         const int cur = it & 1;
         lt_v4f S[2];
+        float ksc[2] = {1.0f, 1.0f};
+        if (p.kscale) {
+            ksc[0] = p.kscale[rowoff[cur * 32 + n]];
+            ksc[1] = p.kscale[rowoff[cur * 32 + 16 + n]];
+        }
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             S[b] = lt_v4f{0, 0, 0, 0};
@@ -477,7 +490,9 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 const int j = kb + 16 * b + n;
-                sv[b] = (j <= pos && j >= lo) ? S[b][g] : -INFINITY;
+                float sc = S[b][g] * ksc[b];
+                if (p.bias) sc += 1.4426950408889634f * p.bias[(int64_t)min(max(pos - j, 0), p.bias_rows - 1) * H + hrow[g]];
+                sv[b] = (j <= pos && j >= lo) ? sc : -INFINITY;
             }
             const float mx = row16_max(fmaxf(sv[0], sv[1]));
             const float mn = fmaxf(mrow[g], mx);
@@ -527,7 +542,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
         const int head = head0 + kg * 4 + g;
-        if (head >= H) continue;
+        if (hin + kg * 4 + g >= rep) continue;
         float* o = p.out + (tok * H + head) * r;
         const float inv = 1.0f / lrow[g];
 #pragma unroll
@@ -618,8 +633,7 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
         I64H_CHECK_ARG(tasks < (1ll << 31), "latent_attn: too many tiles");
         const int splits = (!row_tiles && d.workspace && d.splits > 1) ? (d.splits > 64 ? 64 : d.splits) : 1;
         const size_t bytes = (size_t)d.kv_rank * LT_VLD * 2 + 2 * 16 * LT_VLD * 2 + 64 * 4;
-        const bool plain = G == 1 && d.row_stride <= 0 && d.chunk <= 0 && !d.kscale && !d.bias && !d.sink;   // what the prefetching kernel covers
-        if (row_tiles || !g_decode_form || !plain)
+        if (row_tiles || !g_decode_form)
             hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, row_tiles, splits);
         else
             hipLaunchKernelGGL(latent_attn_mfma_decode_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, splits);

@@ -71,7 +71,7 @@ class _StepBuffers:
 class DogalornModel:
     MAX_BUFFER_SETS = int(os.environ.get("I64H_MAX_BUFFER_SETS", "8"))
     ATTN_MAX_SEGMENTS = 4     # more runs than this in one step (finely interleaved kinds) collapse into one launch
-    ATTN_WAVES = 4096         # waves a decode-sized attention launch aims at (256 CUs, four SIMDs, the kernel keeps two waves each, two turns)
+    ATTN_WAVES = 1024         # waves a decode-sized attention launch aims at (256 CUs, four SIMDs each)
 
     def __init__(self, cfg: DogalornConfig, weights: Dict[str, torch.Tensor], device="cuda:0", dtype: str = "bfloat16", max_seqs: int = 4,
                  num_kv_blocks: int = 256, kv_block: int = 16, cache_dtype: Optional[torch.dtype] = None):
