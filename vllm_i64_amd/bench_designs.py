@@ -266,7 +266,7 @@ def _dogalorn_kernels(sz, rows, batch, ctx, dev):
         q, oa = rn(n, H * dm) * 0.3, torch.empty(n, H * dm, device=dev)
         bias = torch.zeros(sz["chunk"] + 1, H, device=dev)
         keys = seq * (seq + 1) / 2 * nseq if tag == "prefill" else float(min(ctx, sz["chunk"])) * n
-        sp = 1 if tag == "prefill" else max(1, min(1024 // max(1, n * G * ((H // G + 15) // 16)), int(keys / n) // 64, 64))
+        sp = 1 if tag == "prefill" else max(1, min((3072 if dm <= 64 else 1024) // max(1, n * G * ((H // G + 15) // 16)), int(keys / n) // 64, 64))
         t = _time(lambda: D.kattn(q, kc, ks, bt, slots, pos, chunk=sz["chunk"], bias=bias, sink=True, heads=H, kv_heads=G, dim=dm, out=oa, n=n,
                                   mode=3 if tag == "prefill" else 2, splits=sp), reps)
         row(f"kattn_{tag}", t, flops=4.0 * keys * H * dm, bytes_=(2.0 * keys * G * dm if tag == "decode" else 0.0) + 8.0 * n * H * dm)

@@ -536,7 +536,7 @@ int i64h_causal_conv(const i64h_causal_conv_args* dp, void* stream) {
     const dim3 grid((unsigned)((d.channels + 255) / 256), (unsigned)d.n);
     const dim3 walk((unsigned)((d.channels + 255) / 256), (unsigned)((d.n + CV_ROWS - 1) / CV_ROWS));
     hipStream_t s = (hipStream_t)stream;
-    switch (d.n >= 4 * CV_ROWS ? d.taps : 0) {      // few rows: a thread per row and channel fills the chip better
+    switch (d.n >= 32 * CV_ROWS ? d.taps : 0) {     // few rows: a thread per row and channel fills the chip better
         case 2: hipLaunchKernelGGL(causal_conv_walk_kernel<2>, walk, dim3(256), 0, s, d); break;
         case 3: hipLaunchKernelGGL(causal_conv_walk_kernel<3>, walk, dim3(256), 0, s, d); break;
         case 4: hipLaunchKernelGGL(causal_conv_walk_kernel<4>, walk, dim3(256), 0, s, d); break;

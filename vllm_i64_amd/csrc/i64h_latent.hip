@@ -171,7 +171,10 @@ __device__ __forceinline__ void lt_split(float x, uint32_t& hi, uint32_t& lo) {
     lo = lt_rne(x - __uint_as_float(hi << 16));
 }
 
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void latent_attn_mfma_kernel(const i64h_latent_attn_args p, const int row_tiles, const int splits) {
+// KD, NB: 32-wide steps over a cached row and 16-column blocks of the output that the instance holds registers for (rows of at most
+// 32 KD values, kv_rank <= 16 NB): the widest instance keeps two waves per SIMD, narrow rows leave room for more.
+template <int KD, int NB>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, KD > 4 ? 2 : 8))) void latent_attn_mfma_kernel(const i64h_latent_attn_args p, const int row_tiles, const int splits) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x, n = lane & 15, kg = lane >> 4;
     const int r = p.kv_rank, D = r + p.rot_dim, H = p.heads, bs = p.block_size, win = p.window;
@@ -206,12 +209,12 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         info[16 + lane] = valid_n ? p.slot_ids[tok_n] : -1;
     }
     // the query of row n times scale * log2(e) (the softmax runs on powers of two), columns ks * 32 + kg * 8 .. + 7, as two bf16 terms
-    uint4 Qh[LT_KD], Ql[LT_KD];
+    uint4 Qh[KD], Ql[KD];
     {
         const float* q = p.Q + (tok_n * H + head_n) * D;
         const float qs = p.scale * 1.4426950408889634f;
 #pragma unroll
-        for (int ks = 0; ks < LT_KD; ++ks) {
+        for (int ks = 0; ks < KD; ++ks) {
             const int d0 = ks * 32 + kg * 8;
             uint32_t h[8], l[8];
             if (valid_n && d0 < D) {
@@ -227,9 +230,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             Ql[ks] = make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16));
         }
     }
-    lt_v4f acc[LT_NB];
+    lt_v4f acc[NB];
 #pragma unroll
-    for (int nb = 0; nb < LT_NB; ++nb) acc[nb] = lt_v4f{0, 0, 0, 0};
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = lt_v4f{0, 0, 0, 0};
     float mrow[4], lrow[4];
     int lor[4], hrow[4];   // per row of the tile: the first position it sees, its head (for the bias table)
     const bool sink = p.sink && split == 0;     // the extra score of zero counts once: in the first share of the keys
@@ -276,7 +279,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
                 S[b] = lt_v4f{0, 0, 0, 0};
                 const uint16_t* rowp = cache + (int64_t)rowoff[16 * b + n] * rstride + coff;
 #pragma unroll
-                for (int ks = 0; ks < LT_KD; ++ks) {
+                for (int ks = 0; ks < KD; ++ks) {
                     if (ks * 32 < D) {
                         const int d0 = ks * 32 + kg * 8;
                         const uint4 kf = d0 < D ? *(const uint4*)(rowp + d0) : make_uint4(0, 0, 0, 0);
@@ -323,7 +326,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
             __syncthreads();
             const uint4 pah = *(const uint4*)&Ph[n * LT_VLD + kg * 8], pal = *(const uint4*)&Pl[n * LT_VLD + kg * 8];
 #pragma unroll
-            for (int nb = 0; nb < LT_NB; ++nb) {
+            for (int nb = 0; nb < NB; ++nb) {
                 if (nb * 16 < r) {
                     const uint4 vf = *(const uint4*)&Vt[(nb * 16 + n) * LT_VLD + kg * 8];
 #pragma unroll
@@ -343,7 +346,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         for (int g = 0; g < 4; ++g) {
             float* o = w + (kg * 4 + g) * (r + 2);
 #pragma unroll
-            for (int nb = 0; nb < LT_NB; ++nb)
+            for (int nb = 0; nb < NB; ++nb)
                 if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g];
             if (n == 0) {
                 o[r] = mrow[g];
@@ -360,7 +363,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
         float* o = p.out + (tok * H + head) * r;
         const float inv = 1.0f / lrow[g];
 #pragma unroll
-        for (int nb = 0; nb < LT_NB; ++nb)
+        for (int nb = 0; nb < NB; ++nb)
             if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g] * inv;
     }
 }
@@ -370,6 +373,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 // soon as this tile's scores and transposed columns are done - under its softmax and second product - and the cache rows of the tile
 // after that are looked up a tile ahead.  The workgroup is one wave, so LDS traffic needs program order only (no barrier, whose
 // fence would wait for the loads in flight).  Registers: a whole SIMD's (one wave per SIMD is all such a launch has anyway).
+template <int KD, int NB>
 __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_latent_attn_args p, const int splits) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int lane = threadIdx.x, n = lane & 15, kg = lane >> 4;
@@ -400,13 +404,13 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
             rowoff[buf * 32 + lane] = bt[jc / bs] * bs + jc % bs;
         }
     };
-    uint4 kf[2][LT_KD];
+    uint4 kf[2][KD];
     auto request = [&](int buf) {
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             const uint16_t* rowp = cache + (int64_t)rowoff[buf * 32 + 16 * b + n] * rstride + coff;
 #pragma unroll
-            for (int ks = 0; ks < LT_KD; ++ks) {
+            for (int ks = 0; ks < KD; ++ks) {
                 const int d0 = ks * 32 + kg * 8;
                 kf[b][ks] = (ks * 32 < D && d0 < D) ? *(const uint4*)(rowp + d0) : make_uint4(0, 0, 0, 0);
             }
@@ -419,13 +423,13 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
         request(0);
     }
     // the query of row n (head head0 + n) times scale * log2(e), as two bf16 terms - converted while the first tile travels
-    uint4 Qh[LT_KD], Ql[LT_KD];
+    uint4 Qh[KD], Ql[KD];
     {
         const bool valid_n = hin + n < rep;
         const float* q = p.Q + (tok * H + head0 + n) * D;
         const float qs = p.scale * 1.4426950408889634f;
 #pragma unroll
-        for (int ks = 0; ks < LT_KD; ++ks) {
+        for (int ks = 0; ks < KD; ++ks) {
             const int d0 = ks * 32 + kg * 8;
             uint32_t h[8], l[8];
             if (valid_n && d0 < D) {
@@ -441,9 +445,9 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
             Ql[ks] = make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16));
         }
     }
-    lt_v4f acc[LT_NB];
+    lt_v4f acc[NB];
 #pragma unroll
-    for (int nb = 0; nb < LT_NB; ++nb) acc[nb] = lt_v4f{0, 0, 0, 0};
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = lt_v4f{0, 0, 0, 0};
     float mrow[4], lrow[4];
     int hrow[4];
     const bool sink = p.sink && split == 0;     // the extra score of zero counts once: in the first share of the keys
@@ -466,7 +470,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
         for (int b = 0; b < 2; ++b) {
             S[b] = lt_v4f{0, 0, 0, 0};
 #pragma unroll
-            for (int ks = 0; ks < LT_KD; ++ks) {
+            for (int ks = 0; ks < KD; ++ks) {
                 if (ks * 32 < D) {
                     const int d0 = ks * 32 + kg * 8;
                     const uint4 f = kf[b][ks];
@@ -512,7 +516,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
         __builtin_amdgcn_wave_barrier();
         const uint4 pah = *(const uint4*)&Ph[n * LT_VLD + kg * 8], pal = *(const uint4*)&Pl[n * LT_VLD + kg * 8];
 #pragma unroll
-        for (int nb = 0; nb < LT_NB; ++nb) {
+        for (int nb = 0; nb < NB; ++nb) {
             if (nb * 16 < r) {
                 const uint4 vf = *(const uint4*)&Vt[(nb * 16 + n) * LT_VLD + kg * 8];
 #pragma unroll
@@ -530,7 +534,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
         for (int g = 0; g < 4; ++g) {
             float* o = w + (kg * 4 + g) * (r + 2);
 #pragma unroll
-            for (int nb = 0; nb < LT_NB; ++nb)
+            for (int nb = 0; nb < NB; ++nb)
                 if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g];
             if (n == 0) {
                 o[r] = mrow[g];
@@ -546,7 +550,7 @@ __global__ __launch_bounds__(64) void latent_attn_mfma_decode_kernel(const i64h_
         float* o = p.out + (tok * H + head) * r;
         const float inv = 1.0f / lrow[g];
 #pragma unroll
-        for (int nb = 0; nb < LT_NB; ++nb)
+        for (int nb = 0; nb < NB; ++nb)
             if (nb * 16 < r) o[nb * 16 + n] = acc[nb][g] * inv;
     }
 }
@@ -633,10 +637,18 @@ int i64h_latent_attn(const i64h_latent_attn_args* dp, void* stream) {
         I64H_CHECK_ARG(tasks < (1ll << 31), "latent_attn: too many tiles");
         const int splits = (!row_tiles && d.workspace && d.splits > 1) ? (d.splits > 64 ? 64 : d.splits) : 1;
         const size_t bytes = (size_t)d.kv_rank * LT_VLD * 2 + 2 * 16 * LT_VLD * 2 + 64 * 4;
-        if (row_tiles || !g_decode_form)
-            hipLaunchKernelGGL(latent_attn_mfma_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, row_tiles, splits);
-        else
-            hipLaunchKernelGGL(latent_attn_mfma_decode_kernel, dim3((unsigned)tasks, (unsigned)splits), dim3(64), bytes, (hipStream_t)stream, d, splits);
+        const dim3 grid((unsigned)tasks, (unsigned)splits);
+        hipStream_t st = (hipStream_t)stream;
+        const int size = (D <= 64 && d.kv_rank <= 64) ? 0 : ((D <= 128 && d.kv_rank <= 128) ? 1 : 2);     // the narrowest instance that holds the rows
+        if (row_tiles || !g_decode_form) {
+            if (size == 0) hipLaunchKernelGGL((latent_attn_mfma_kernel<2, 4>), grid, dim3(64), bytes, st, d, row_tiles, splits);
+            else if (size == 1) hipLaunchKernelGGL((latent_attn_mfma_kernel<4, 8>), grid, dim3(64), bytes, st, d, row_tiles, splits);
+            else hipLaunchKernelGGL((latent_attn_mfma_kernel<LT_KD, LT_NB>), grid, dim3(64), bytes, st, d, row_tiles, splits);
+        } else {
+            if (size == 0) hipLaunchKernelGGL((latent_attn_mfma_decode_kernel<2, 4>), grid, dim3(64), bytes, st, d, splits);
+            else if (size == 1) hipLaunchKernelGGL((latent_attn_mfma_decode_kernel<4, 8>), grid, dim3(64), bytes, st, d, splits);
+            else hipLaunchKernelGGL((latent_attn_mfma_decode_kernel<LT_KD, LT_NB>), grid, dim3(64), bytes, st, d, splits);
+        }
         I64H_CHECK_LAUNCH();
         if (splits > 1) {
             hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)tasks, 16), dim3(64), 0, (hipStream_t)stream, d, splits);

@@ -71,7 +71,8 @@ class _StepBuffers:
 class DogalornModel:
     MAX_BUFFER_SETS = int(os.environ.get("I64H_MAX_BUFFER_SETS", "8"))
     ATTN_MAX_SEGMENTS = 4     # more runs than this in one step (finely interleaved kinds) collapse into one launch
-    ATTN_WAVES = 1024         # waves a decode-sized attention launch aims at (256 CUs, four SIMDs each)
+    ATTN_WAVES = {64: 3072, 128: 2048, 256: 1024}     # waves a decode-sized attention launch aims at, by head size: 1024 SIMDs, and the
+                                                      # kernel's instance for narrow rows leaves registers for three waves on each
 
     def __init__(self, cfg: DogalornConfig, weights: Dict[str, torch.Tensor], device="cuda:0", dtype: str = "bfloat16", max_seqs: int = 4,
                  num_kv_blocks: int = 256, kv_block: int = 16, cache_dtype: Optional[torch.dtype] = None):
@@ -243,7 +244,8 @@ class DogalornModel:
             if one_per_seq and not ex:
                 keys = min(a.chunk, ctx_hint) if a.chunk > 0 else ctx_hint
                 tasks = (r1 - r0) * a.kv_heads * ((a.heads // a.kv_heads + 15) // 16)
-                splits = max(1, min(self.ATTN_WAVES // max(1, tasks), keys // 64, 64))
+                waves = self.ATTN_WAVES[64 if a.dim <= 64 else (128 if a.dim <= 128 else 256)]
+                splits = max(1, min(waves // max(1, tasks), keys // 64, 64))
                 if splits > 1:
                     key = (r1 - r0, a.heads, a.kv_heads, a.dim, splits)
                     ws = B.attn_ws.get(key)
