@@ -261,7 +261,7 @@ def test_streams_write_and_read(dev, S, W):
         assert close(st, xs + y, 1e-6)
 
 
-def _mamba_case(dev, heads, vdim, state, groups, conv, norm_groups, cut_sizes, seed):
+def _mamba_case(dev, heads, vdim, state, groups, conv, norm_groups, cut_sizes, seed, lens=None):
     """The state-space mixer from its in-projection's output on: convolution, recurrence, gate and norm; two sequences in slots 3 and 1,
     cut into portions, against the oracle (whose out-projection is the identity here)."""
     from vllm_i64_amd import ops_dense as D
@@ -273,7 +273,7 @@ def _mamba_case(dev, heads, vdim, state, groups, conv, norm_groups, cut_sizes, s
          "dt_bias": torch.rand(heads, generator=g) * 3 - 2, "A_log": torch.rand(heads, generator=g) * 2.5 - 1.5, "D": torch.rand(heads, generator=g) + 0.5,
          "norm": torch.rand(inner, generator=g) + 0.5, "o": torch.eye(inner)}
     eps = 1e-5
-    lens = {3: 150, 1: 70}
+    lens = lens or {3: 150, 1: 70}
     proj = {s: torch.randn(T, nin, generator=g) for s, T in lens.items()}
     want = {s: R.mamba2({k: v.double() for k, v in w.items()}, "", m, eps, proj[s].double()) for s in lens}
     cw, cb = w["conv"].to(dev), w["conv.b"].to(dev)
@@ -305,6 +305,13 @@ def test_mamba2_mechanism_under_cuts(dev, cut_sizes):
     _mamba_case(dev, heads=1, vdim=3, state=130, groups=1, conv=1, norm_groups=3, cut_sizes=cut_sizes, seed=3)
     _mamba_case(dev, heads=2, vdim=20, state=32, groups=2, conv=8, norm_groups=1, cut_sizes=cut_sizes, seed=4)
     _mamba_case(dev, heads=1, vdim=17, state=7, groups=1, conv=11, norm_groups=1, cut_sizes=cut_sizes, seed=5)
+
+
+@pytest.mark.parametrize("conv", [2, 4, 7, 8])
+def test_mamba2_mechanism_long_launches(dev, conv):
+    """Launches of 512 rows and more (the convolution then walks 16 rows per thread), runs that start and end inside a walk."""
+    for cut_sizes in ([700], [523, 1, 40]):
+        _mamba_case(dev, heads=2, vdim=5, state=4, groups=1, conv=conv, norm_groups=1, cut_sizes=cut_sizes, seed=conv, lens={3: 571, 1: 90, 0: 7})
 
 
 @pytest.mark.parametrize("cut_sizes", [[200], [1], [2, 9, 1, 30]])
