@@ -89,7 +89,7 @@ class DogalornModel:
         def need(name, shape):
             if name not in weights:
                 raise KeyError(f"tensor '{name}' is missing")
-            if tuple(weights[name].shape) != tuple(shape):
+            if tuple(weights[name].shape) != tuple(shape) and not (tuple(shape) == () and weights[name].numel() == 1):     # (a single number, however it is stored)
                 raise ValueError(f"'{name}': shape {tuple(weights[name].shape)}, config says {tuple(shape)}")
             return weights[name]
 
